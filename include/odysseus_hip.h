@@ -1,0 +1,164 @@
+/*
+ * odysseus_hip.h -- C ABI of libodysseus_hip.so: the per-rank compute of the
+ * Odysseus decoder layer as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The reference has no FFI layer: its boundary is Python (nn.Module classes and
+ * torch.autograd.Function.apply) over third-party kernels.  Each entry point
+ * below replaces the third-party routine that a reference call site invokes;
+ * the call site is cited next to it.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; the library never
+ *     allocates, frees or keeps a pointer after the call returns;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); no entry
+ *     point synchronises the device;
+ *   - `dtype` is ODY_BF16 (bf16 storage, fp32 accumulation, MFMA) or ODY_F32
+ *     (fp32 storage and arithmetic);
+ *   - strides are in ELEMENTS; the innermost (head_dim / feature) stride is 1;
+ *   - return value: 0 on success, a negative ody_status otherwise;
+ *     ody_last_error() returns a thread-local message for the last failure.
+ *     Nothing throws or aborts across this boundary.
+ */
+#ifndef ODYSSEUS_HIP_H
+#define ODYSSEUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum ody_dtype { ODY_BF16 = 0, ODY_F32 = 1 };
+
+enum ody_status {
+  ODY_OK = 0,
+  ODY_ERR_BAD_SHAPE = -1,      /* non-positive size, Hq % Hkv != 0, ... */
+  ODY_ERR_UNSUPPORTED = -2,    /* head_dim / dtype / flag combination not built */
+  ODY_ERR_MISALIGNED = -3,     /* pointer or stride breaks the 16-byte rule */
+  ODY_ERR_NULL = -4,           /* required pointer is NULL */
+  ODY_ERR_WORKSPACE = -5,      /* workspace smaller than ody_*_workspace_bytes */
+  ODY_ERR_LAUNCH = -6          /* hipLaunchKernel reported an error */
+};
+
+const char* ody_last_error(void);
+int ody_version(void);
+
+/* ---- attention ---------------------------------------------------------
+ * Replaces flash_attn_func(q, k, v, dropout_p=0, softmax_scale, causal) as
+ * reached from decoder/odysseus.py:256-263 (via HF _flash_attention_forward),
+ * and the per-block attention of the ring step entered at decoder/ring.py:30-37.
+ *
+ * q   (B, Lq, Hq,  D)  strides sq_b, sq_l, sq_h   (head-axis slices of the packed
+ * k,v (B, Lk, Hkv, D)  strides sk_*, sv_*          QKV buffer are accepted as is)
+ * out (B, Lq, Hq,  D)  strides so_*
+ * lse (B, Hq, Lq) fp32 contiguous, natural-log units; -inf for a query row that
+ *                      sees no key (its out row is 0).
+ * GQA: q head h reads kv head h / (Hq / Hkv).  causal != 0 masks key j for
+ * query i when j > i + (Lk - Lq).  D in {64, 128}.
+ */
+int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                 int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                 int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                 int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                 int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                 int64_t so_b, int64_t so_l, int64_t so_h,
+                 float scale, int causal, int dtype, void* stream);
+
+/* Backward of the above (flash_attn's backward as run by autograd through
+ * decoder/odysseus.py:256-263).  `out` and `lse` are the forward results -- or,
+ * for a ring step, the FINAL merged out / lse, which is what makes the per-block
+ * gradients sum to the gradient of the unsplit attention.
+ * dq/dk/dv have the shapes of q/k/v with their own strides.  dK and dV of a kv
+ * head are summed over its query-head group inside the kernel (deterministic,
+ * no atomics).  If accumulate_dq != 0 the kernel adds into dq (fp32 dq_accum
+ * layout not needed: the add happens in fp32 before rounding once).
+ * workspace: ody_attn_bwd_workspace_bytes(B, Lq, Hq) bytes, 256-byte aligned.
+ */
+size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Hq);
+int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                 const void* dout, void* dq, void* dk, void* dv,
+                 int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                 int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                 int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                 int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                 int64_t so_b, int64_t so_l, int64_t so_h,
+                 int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                 int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                 int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                 int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                 float scale, int causal, int accumulate_dq, int dtype,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* Online-softmax merge of one key block's partial result into the running one
+ * (the update rule of ring_flash_attn, reached from decoder/ring.py:30-37):
+ *   lse' = logaddexp(lse, lse_blk)
+ *   out' = out * e^(lse - lse') + out_blk * e^(lse_blk - lse')
+ * out_acc (B, L, H, D) fp32 contiguous, updated in place; lse_acc (B, H, L) fp32
+ * updated in place; out_blk (B, L, H, D) of `dtype` with strides sb_*; lse_blk
+ * (B, H, L) fp32.  A side whose lse is -inf contributes nothing.
+ */
+int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk, const float* lse_blk,
+                  int B, int L, int H, int D, int64_t sb_b, int64_t sb_l, int64_t sb_h,
+                  int dtype, void* stream);
+
+/* ---- dense linears ------------------------------------------------------
+ * C (M, N) = op(A) * op(B), row-major, leading dimensions in elements.
+ *   ODY_GEMM_NT  C = A (M,K) * B (N,K)^T   forward  X W^T   utils/linear_tpsp.py:173,
+ *                                                           :588, utils/linear_zero3.py:44
+ *   ODY_GEMM_NN  C = A (M,K) * B (K,N)     dgrad    dY W    utils/linear_tpsp.py:217,
+ *                                                           utils/linear_zero3.py:68
+ *   ODY_GEMM_TN  C = A (K,M)^T * B (K,N)   wgrad    dY^T X  utils/linear_tpsp.py:291,
+ *                                                           utils/linear_zero3.py:74
+ * bias (N) of `dtype` or NULL is added to every row (utils/linear_tpsp.py:175-176).
+ * If accumulate != 0, C += result (C read in `dtype`, added in fp32).
+ */
+enum ody_gemm_op { ODY_GEMM_NT = 0, ODY_GEMM_NN = 1, ODY_GEMM_TN = 2 };
+int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias,
+             int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+             int accumulate, int dtype, void* stream);
+
+/* ---- SwiGLU -------------------------------------------------------------
+ * decoder/odysseus.py:293-295: a1, a3 = gate_up.chunk(2, -1); h = silu(a1) * a3.
+ * gate_up (T, 2*I) row stride ld_gu; h (T, I) row stride ld_h.
+ * bwd: d_gate_up (T, 2*I) from gate_up and dh.
+ */
+int ody_swiglu_fwd(const void* gate_up, void* h, int T, int I, int64_t ld_gu, int64_t ld_h,
+                   int dtype, void* stream);
+int ody_swiglu_bwd(const void* gate_up, const void* dh, void* d_gate_up, int T, int I,
+                   int64_t ld_gu, int64_t ld_dh, int64_t ld_dgu, int dtype, void* stream);
+
+/* ---- RMSNorm ------------------------------------------------------------
+ * HF LlamaRMSNorm as called by the decoder layer (decoder/ring.py:67,84):
+ * y = w * (x * rsqrt(mean(x^2) + eps)) with fp32 statistics.  x, y (T, d)
+ * contiguous; rstd (T) fp32 is written by fwd and read by bwd.
+ * bwd: dx (T, d); dw_partial (n_partial, d) fp32 partial column sums, where
+ * n_partial = ody_rmsnorm_bwd_partials(T); the caller (or ody_rmsnorm_bwd with
+ * dw != NULL) reduces them: dw (d) of `dtype`.
+ */
+int ody_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int T, int d, float eps,
+                    int dtype, void* stream);
+int ody_rmsnorm_bwd_partials(int T);
+int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
+                    float* dw_partial, void* dw, int T, int d, int dtype, void* stream);
+
+/* ---- RoPE ---------------------------------------------------------------
+ * HF rotary_emb + apply_rotary_pos_emb at decoder/odysseus.py:210-213
+ * (half-rotation convention; angles computed in fp32 from position * base^(-2j/D),
+ * cos/sin rounded to `dtype` before use, as HF does).
+ * x (B, L, H, D) with strides sx_*, rotated IN PLACE for the first n_rot heads on
+ * the head axis (q and k heads of the packed buffer are adjacent, v is left alone).
+ * position_ids (B, L) int64 or NULL for arange(L).  inv_freq (D/2) fp32 is the
+ * frequency table base^(-2j/D) as the caller's rotary module holds it (passing
+ * the table keeps the angles bit-identical to the host's and admits scaled
+ * variants); NULL evaluates base^(-2j/D) in the kernel.  inverse != 0 rotates by
+ * the opposite angle (the backward pass).
+ */
+int ody_rope(void* x, const int64_t* position_ids, const float* inv_freq, int B, int L, int n_rot,
+             int D, int64_t sx_b, int64_t sx_l, int64_t sx_h, float base, int inverse,
+             int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ODYSSEUS_HIP_H */

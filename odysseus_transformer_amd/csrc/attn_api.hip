@@ -1,0 +1,136 @@
+// extern "C" entry points for attention and the error channel of the library.
+#include <cstdarg>
+#include <cstdio>
+#include <cmath>
+#include "attn_params.h"
+
+namespace {
+thread_local char g_err[512] = "";
+}
+
+void ody_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int ody_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    ody_set_error("%s: launch failed: %s", what, hipGetErrorString(e));
+    return ODY_ERR_LAUNCH;
+  }
+  return ODY_OK;
+}
+
+extern "C" const char* ody_last_error(void) { return g_err; }
+extern "C" int ody_version(void) { return 1; }
+
+namespace {
+
+int check_common(const char* who, int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
+  ODY_REQUIRE(B > 0 && Lq > 0 && Lk > 0 && Hq > 0 && Hkv > 0, ODY_ERR_BAD_SHAPE,
+              "%s: sizes must be positive (B=%d Lq=%d Lk=%d Hq=%d Hkv=%d)", who, B, Lq, Lk, Hq, Hkv);
+  ODY_REQUIRE(Hq % Hkv == 0, ODY_ERR_BAD_SHAPE, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
+  ODY_REQUIRE(D == 64 || D == 128, ODY_ERR_UNSUPPORTED, "%s: head_dim %d not built (64, 128)", who, D);
+  ODY_REQUIRE(dtype == ODY_BF16 || dtype == ODY_F32, ODY_ERR_UNSUPPORTED, "%s: dtype %d unknown", who, dtype);
+  ODY_REQUIRE(B <= 65535 && Hq <= 65535, ODY_ERR_BAD_SHAPE, "%s: B and Hq must fit a grid dimension", who);
+  return ODY_OK;
+}
+
+// The MFMA kernels move 16-byte vectors: pointers 16-byte aligned, strides multiples of 8 elements.
+// The fp32 kernels use scalar accesses except for the delta pre-pass (16-byte vectors of 4 floats).
+int check_tensor(const char* who, const char* name, const void* ptr, const AttnStrides& s, int dtype, bool vec) {
+  ODY_REQUIRE(ptr != nullptr, ODY_ERR_NULL, "%s: %s is NULL", who, name);
+  if (vec) {
+    const int q = (dtype == ODY_BF16) ? 8 : 4;
+    ODY_REQUIRE(ody_aligned16(ptr) && s.b % q == 0 && s.l % q == 0 && s.h % q == 0, ODY_ERR_MISALIGNED,
+                "%s: %s needs a 16-byte aligned pointer and strides that are multiples of %d elements", who, name, q);
+  }
+  return ODY_OK;
+}
+
+}  // namespace
+
+extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                            int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                            int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                            int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                            int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                            int64_t so_b, int64_t so_l, int64_t so_h,
+                            float scale, int causal, int dtype, void* stream) {
+  int rc = check_common("ody_attn_fwd", B, Lq, Lk, Hq, Hkv, D, dtype);
+  if (rc) return rc;
+  AttnParams p{};
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
+  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.causal = causal ? 1 : 0; p.off = Lk - Lq;
+  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
+  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
+  const bool vec = (dtype == ODY_BF16);
+  if ((rc = check_tensor("ody_attn_fwd", "q", q, p.sq, dtype, vec))) return rc;
+  if ((rc = check_tensor("ody_attn_fwd", "k", k, p.sk, dtype, vec))) return rc;
+  if ((rc = check_tensor("ody_attn_fwd", "v", v, p.sv, dtype, vec))) return rc;
+  if ((rc = check_tensor("ody_attn_fwd", "out", out, p.so, dtype, vec))) return rc;
+  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_fwd: lse is NULL");
+  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_fwd: scale must be positive");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
+  return ody_launch_attn_fwd_simt(p, D, dtype, st);
+}
+
+extern "C" size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Hq) {
+  if (B <= 0 || Lq <= 0 || Hq <= 0) return 0;
+  const size_t n = (size_t)B * Lq * Hq * sizeof(float);
+  return (n + 255) & ~(size_t)255;
+}
+
+extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                            const void* dout, void* dq, void* dk, void* dv,
+                            int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                            int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                            int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                            int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                            int64_t so_b, int64_t so_l, int64_t so_h,
+                            int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                            int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                            int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                            int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                            float scale, int causal, int accumulate_dq, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_common("ody_attn_bwd", B, Lq, Lk, Hq, Hkv, D, dtype);
+  if (rc) return rc;
+  AttnParams p{};
+  p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
+  p.dout = dout; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.causal = causal ? 1 : 0; p.off = Lk - Lq; p.accumulate_dq = accumulate_dq ? 1 : 0;
+  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
+  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
+  p.sdo = {sdo_b, sdo_l, sdo_h}; p.sdq = {sdq_b, sdq_l, sdq_h}; p.sdk = {sdk_b, sdk_l, sdk_h};
+  p.sdv = {sdv_b, sdv_l, sdv_h};
+  const bool vec = (dtype == ODY_BF16);
+  const char* who = "ody_attn_bwd";
+  if ((rc = check_tensor(who, "q", q, p.sq, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "k", k, p.sk, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "out", out, p.so, dtype, true))) return rc;    // delta pre-pass is vectorised
+  if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, true))) return rc;
+  if ((rc = check_tensor(who, "dq", dq, p.sdq, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dk", dk, p.sdk, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dv", dv, p.sdv, dtype, vec))) return rc;
+  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_bwd: lse is NULL");
+  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_bwd: scale must be positive");
+  ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_bwd: workspace is NULL");
+  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Hq), ODY_ERR_WORKSPACE,
+              "ody_attn_bwd: workspace of %zu bytes, %zu needed", workspace_bytes,
+              ody_attn_bwd_workspace_bytes(B, Lq, Hq));
+  ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
+              "ody_attn_bwd: workspace must be 256-byte aligned");
+  p.delta = static_cast<float*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if ((rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
+  if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
+  return ody_launch_attn_bwd_simt(p, D, dtype, st);
+}

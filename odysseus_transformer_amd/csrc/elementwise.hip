@@ -1,0 +1,445 @@
+// Memory-bound kernels of the decoder layer: RMSNorm, RoPE, SwiGLU, LSE merge.
+// All move 16-byte vectors per lane, keep statistics in fp32 and reduce inside a
+// wavefront with lane shuffles; none of them is shaped into a matrix product.
+#include <cmath>
+#include "ody_common.h"
+
+namespace {
+
+template <typename T> struct VecIO {
+  static constexpr int N = Vec16B<T>::N;
+  typedef typename Vec16B<T>::type vec_t;
+  __device__ static __forceinline__ void load(const T* p, float (&f)[N]) {
+    const vec_t v = *reinterpret_cast<const vec_t*>(p);
+#pragma unroll
+    for (int e = 0; e < N; e++) f[e] = (float)v[e];
+  }
+  __device__ static __forceinline__ void store(T* p, const float (&f)[N]) {
+    vec_t v;
+#pragma unroll
+    for (int e = 0; e < N; e++) v[e] = (T)f[e];
+    *reinterpret_cast<vec_t*>(p) = v;
+  }
+};
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) x += __shfl_xor(x, s, 64);
+  return x;
+}
+
+// round-trip through the storage type (a no-op for fp32)
+template <typename T> __device__ __forceinline__ float rnd(float x) { return (float)(T)x; }
+
+// ---------------------------------------------------------------------------
+// RMSNorm forward: one wavefront per row; the row is cached in registers when it
+// fits (d <= 64 * N * CACHE), otherwise re-read.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          T* __restrict__ y, float* __restrict__ rstd_out, int Trows,
+                                                          int d, float eps) {
+  constexpr int N = VecIO<T>::N, CACHE = 8;
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= Trows) return;
+  const T* xr = x + (int64_t)row * d;
+  T* yr = y + (int64_t)row * d;
+  const int nvec = d / N;
+  float cache[CACHE][N];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CACHE; c++) {
+    const int vi = lane + 64 * c;
+    if (vi < nvec) {
+      VecIO<T>::load(xr + vi * N, cache[c]);
+#pragma unroll
+      for (int e = 0; e < N; e++) ss = fmaf(cache[c][e], cache[c][e], ss);
+    }
+  }
+  for (int vi = lane + 64 * CACHE; vi < nvec; vi += 64) {
+    float f[N];
+    VecIO<T>::load(xr + vi * N, f);
+#pragma unroll
+    for (int e = 0; e < N; e++) ss = fmaf(f[e], f[e], ss);
+  }
+  ss = wave_sum(ss);
+  const float rstd = rsqrtf(ss / (float)d + eps);
+  if (lane == 0 && rstd_out) rstd_out[row] = rstd;
+#pragma unroll
+  for (int c = 0; c < CACHE; c++) {
+    const int vi = lane + 64 * c;
+    if (vi < nvec) {
+      float wf[N], o[N];
+      VecIO<T>::load(w + vi * N, wf);
+#pragma unroll
+      for (int e = 0; e < N; e++) o[e] = wf[e] * rnd<T>(cache[c][e] * rstd);
+      VecIO<T>::store(yr + vi * N, o);
+    }
+  }
+  for (int vi = lane + 64 * CACHE; vi < nvec; vi += 64) {
+    float f[N], wf[N], o[N];
+    VecIO<T>::load(xr + vi * N, f);
+    VecIO<T>::load(w + vi * N, wf);
+#pragma unroll
+    for (int e = 0; e < N; e++) o[e] = wf[e] * rnd<T>(f[e] * rstd);
+    VecIO<T>::store(yr + vi * N, o);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm backward.  A block owns a contiguous range of rows; for each row its
+// 4 wavefronts compute c = mean(g * xhat) (g = dy * w) and write
+// dx = rstd * (g - xhat * c); every lane also accumulates dy * xhat for its own
+// columns, written at the end as one row of the fp32 partial-sum matrix.
+// ---------------------------------------------------------------------------
+constexpr int RMS_BWD_MAXK = 4;  // column vectors per lane: d <= 256 * N * MAXK
+
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                          const float* __restrict__ rstd, const T* __restrict__ dy,
+                                                          T* __restrict__ dx, float* __restrict__ dw_partial,
+                                                          int Trows, int d, int rows_per_block) {
+  constexpr int N = VecIO<T>::N, MAXK = RMS_BWD_MAXK;
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nvec = d / N;
+  const int r0 = blockIdx.x * rows_per_block, r1 = min(Trows, r0 + rows_per_block);
+  float wf[MAXK][N], acc[MAXK][N];
+#pragma unroll
+  for (int k = 0; k < MAXK; k++) {
+    const int vi = tid + 256 * k;
+#pragma unroll
+    for (int e = 0; e < N; e++) acc[k][e] = 0.f, wf[k][e] = 0.f;
+    if (vi < nvec) VecIO<T>::load(w + vi * N, wf[k]);
+  }
+  for (int row = r0; row < r1; row++) {
+    const float rs = rstd[row];
+    float xh[MAXK][N], gv[MAXK][N];
+    float part = 0.f;
+#pragma unroll
+    for (int k = 0; k < MAXK; k++) {
+      const int vi = tid + 256 * k;
+      if (vi < nvec) {
+        float dyv[N];
+        VecIO<T>::load(x + (int64_t)row * d + vi * N, xh[k]);
+        VecIO<T>::load(dy + (int64_t)row * d + vi * N, dyv);
+#pragma unroll
+        for (int e = 0; e < N; e++) {
+          xh[k][e] *= rs;
+          gv[k][e] = dyv[e] * wf[k][e];
+          part = fmaf(gv[k][e], xh[k][e], part);
+          acc[k][e] = fmaf(dyv[e], xh[k][e], acc[k][e]);
+        }
+      }
+    }
+    part = wave_sum(part);
+    const int pb = (row - r0) & 1;  // alternate slots so that one barrier per row suffices
+    if (lane == 0) red[pb][wave] = part;
+    __syncthreads();
+    const float c = (red[pb][0] + red[pb][1] + red[pb][2] + red[pb][3]) / (float)d;
+#pragma unroll
+    for (int k = 0; k < MAXK; k++) {
+      const int vi = tid + 256 * k;
+      if (vi < nvec) {
+        float o[N];
+#pragma unroll
+        for (int e = 0; e < N; e++) o[e] = rs * (gv[k][e] - xh[k][e] * c);
+        VecIO<T>::store(dx + (int64_t)row * d + vi * N, o);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < MAXK; k++) {
+    const int vi = tid + 256 * k;
+    if (vi < nvec) {
+#pragma unroll
+      for (int e = 0; e < N; e++) dw_partial[(int64_t)blockIdx.x * d + vi * N + e] = acc[k][e];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, T* __restrict__ out, int n,
+                                                     int d) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= d) return;
+  float s = 0.f;
+  for (int r = 0; r < n; r++) s += partial[(int64_t)r * d + c];
+  out[c] = (T)s;
+}
+
+// ---------------------------------------------------------------------------
+// RoPE, half-rotation convention, in place.  A thread owns N frequency indices
+// j..j+N-1 of one (batch, position), evaluates cos/sin once and walks over the
+// heads: x[j] <- x[j]*c - x[j+D/2]*s ; x[j+D/2] <- x[j+D/2]*c + x[j]*s
+// (inverse: s -> -s).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kernel(T* __restrict__ x, const int64_t* __restrict__ pos_ids,
+                                                   const float* __restrict__ inv_freq, int B, int L, int n_rot, int D,
+                                                   int64_t sb, int64_t sl, int64_t sh, float log2_base, int inverse) {
+  constexpr int N = VecIO<T>::N;
+  const int half = D / 2, vph = half / N;  // vectors per half row
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)B * L * vph) return;
+  const int jv = idx % vph;
+  const int l = (idx / vph) % L;
+  const int b = idx / ((int64_t)vph * L);
+  const float pos = pos_ids ? (float)pos_ids[(int64_t)b * L + l] : (float)l;
+  float cs[N], sn[N];
+#pragma unroll
+  for (int e = 0; e < N; e++) {
+    const int j = jv * N + e;
+    const float f = inv_freq ? inv_freq[j] : exp2f(-(2.0f * j / D) * log2_base);
+    const float th = pos * f;
+    // cos/sin are rounded to the storage type before use, as the caller of the
+    // replaced routine does (cos.to(dtype), sin.to(dtype))
+    cs[e] = rnd<T>(cosf(th));
+    sn[e] = rnd<T>(sinf(th));
+    if (inverse) sn[e] = -sn[e];
+  }
+  T* base = x + b * sb + (int64_t)l * sl + jv * N;
+  for (int h = 0; h < n_rot; h++) {
+    T* p1 = base + h * sh;
+    T* p2 = p1 + half;
+    float a[N], c[N], o1[N], o2[N];
+    VecIO<T>::load(p1, a);
+    VecIO<T>::load(p2, c);
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      o1[e] = a[e] * cs[e] - c[e] * sn[e];
+      o2[e] = c[e] * cs[e] + a[e] * sn[e];
+    }
+    VecIO<T>::store(p1, o1);
+    VecIO<T>::store(p2, o2);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, int Trows, int I,
+                                                         int64_t ld_gu, int64_t ld_h) {
+  constexpr int N = VecIO<T>::N;
+  const int vpr = I / N;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)Trows * vpr) return;
+  const int jv = idx % vpr;
+  const int64_t t = idx / vpr;
+  float a1[N], a3[N], o[N];
+  VecIO<T>::load(gu + t * ld_gu + jv * N, a1);
+  VecIO<T>::load(gu + t * ld_gu + I + jv * N, a3);
+#pragma unroll
+  for (int e = 0; e < N; e++) o[e] = a1[e] / (1.f + __expf(-a1[e])) * a3[e];
+  VecIO<T>::store(h + t * ld_h + jv * N, o);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ gu, const T* __restrict__ dh,
+                                                         T* __restrict__ dgu, int Trows, int I, int64_t ld_gu,
+                                                         int64_t ld_dh, int64_t ld_dgu) {
+  constexpr int N = VecIO<T>::N;
+  const int vpr = I / N;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)Trows * vpr) return;
+  const int jv = idx % vpr;
+  const int64_t t = idx / vpr;
+  float a1[N], a3[N], g[N], d1[N], d3[N];
+  VecIO<T>::load(gu + t * ld_gu + jv * N, a1);
+  VecIO<T>::load(gu + t * ld_gu + I + jv * N, a3);
+  VecIO<T>::load(dh + t * ld_dh + jv * N, g);
+#pragma unroll
+  for (int e = 0; e < N; e++) {
+    const float sig = 1.f / (1.f + __expf(-a1[e]));
+    d1[e] = g[e] * a3[e] * sig * (1.f + a1[e] * (1.f - sig));
+    d3[e] = g[e] * a1[e] * sig;
+  }
+  VecIO<T>::store(dgu + t * ld_dgu + jv * N, d1);
+  VecIO<T>::store(dgu + t * ld_dgu + I + jv * N, d3);
+}
+
+// ---------------------------------------------------------------------------
+// LSE merge: 4 head-dim elements per lane, D/4 lanes per (b, l, h) row.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void lse_merge_kernel(float* __restrict__ out_acc, float* __restrict__ lse_acc,
+                                                        const T* __restrict__ out_blk,
+                                                        const float* __restrict__ lse_blk, int B, int L, int H, int D,
+                                                        int64_t sb, int64_t sl, int64_t sh) {
+  const int lpr = D / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)B * L * H * lpr) return;
+  const int sub = idx % lpr;
+  const int64_t row = idx / lpr;  // (b, l, h) order
+  const int h = row % H;
+  const int l = (row / H) % L;
+  const int b = row / ((int64_t)H * L);
+  const int64_t li = ((int64_t)b * H + h) * L + l;
+  const float a = lse_acc[li], c = lse_blk[li];
+  const float mx = fmaxf(a, c);
+  float nw, wa, wb;
+  if (mx == -INFINITY) {
+    nw = -INFINITY, wa = 0.f, wb = 0.f;
+  } else {
+    nw = mx + logf(expf(a - mx) + expf(c - mx));
+    wa = expf(a - nw), wb = expf(c - nw);
+  }
+  float* oa = out_acc + row * D + sub * 4;
+  const T* ob = out_blk + b * sb + (int64_t)l * sl + h * sh + sub * 4;
+  f32x4 va = *reinterpret_cast<const f32x4*>(oa);
+  float vb[4];
+  if constexpr (sizeof(T) == 2) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(ob);
+#pragma unroll
+    for (int e = 0; e < 4; e++) vb[e] = (float)t[e];
+  } else {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(ob);
+#pragma unroll
+    for (int e = 0; e < 4; e++) vb[e] = t[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) va[e] = va[e] * wa + vb[e] * wb;
+  *reinterpret_cast<f32x4*>(oa) = va;
+  // every lane of this row sits in one wavefront and has read lse_acc above
+  if (sub == 0) lse_acc[li] = nw;
+}
+
+inline unsigned blocks_for(int64_t n) { return (unsigned)((n + 255) / 256); }
+
+template <typename T> constexpr int vecn() { return Vec16B<T>::N; }
+
+}  // namespace
+
+#define ODY_BY_DTYPE(dtype, EXPR_BF16, EXPR_F32)                         \
+  if ((dtype) == ODY_BF16) { EXPR_BF16; }                                \
+  else if ((dtype) == ODY_F32) { EXPR_F32; }                             \
+  else { ody_set_error("dtype %d unknown", (dtype)); return ODY_ERR_UNSUPPORTED; }
+
+extern "C" int ody_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int T, int d, float eps, int dtype,
+                               void* stream) {
+  ODY_REQUIRE(x && w && y, ODY_ERR_NULL, "ody_rmsnorm_fwd: NULL pointer");
+  ODY_REQUIRE(T > 0 && d > 0, ODY_ERR_BAD_SHAPE, "ody_rmsnorm_fwd: T=%d d=%d", T, d);
+  const int n = dtype == ODY_BF16 ? 8 : 4;
+  ODY_REQUIRE(d % n == 0, ODY_ERR_UNSUPPORTED, "ody_rmsnorm_fwd: d=%d must be a multiple of %d", d, n);
+  ODY_REQUIRE(ody_aligned16(x) && ody_aligned16(w) && ody_aligned16(y), ODY_ERR_MISALIGNED,
+              "ody_rmsnorm_fwd: pointers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  dim3 grid((T + 3) / 4);
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(rmsnorm_fwd_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
+                                  (bf16*)y, rstd, T, d, eps),
+               hipLaunchKernelGGL(rmsnorm_fwd_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)w,
+                                  (float*)y, rstd, T, d, eps));
+  return ody_check_launch("rmsnorm_fwd");
+}
+
+extern "C" int ody_rmsnorm_bwd_partials(int T) { return T <= 0 ? 0 : (T < 512 ? T : 512); }
+
+extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
+                               float* dw_partial, void* dw, int T, int d, int dtype, void* stream) {
+  ODY_REQUIRE(x && w && rstd && dy && dx && dw_partial, ODY_ERR_NULL, "ody_rmsnorm_bwd: NULL pointer");
+  ODY_REQUIRE(T > 0 && d > 0, ODY_ERR_BAD_SHAPE, "ody_rmsnorm_bwd: T=%d d=%d", T, d);
+  const int n = dtype == ODY_BF16 ? 8 : 4;
+  ODY_REQUIRE(d % n == 0 && d <= 256 * n * RMS_BWD_MAXK, ODY_ERR_UNSUPPORTED,
+              "ody_rmsnorm_bwd: d=%d must be a multiple of %d and at most %d", d, n, 256 * n * RMS_BWD_MAXK);
+  ODY_REQUIRE(ody_aligned16(x) && ody_aligned16(w) && ody_aligned16(dy) && ody_aligned16(dx), ODY_ERR_MISALIGNED,
+              "ody_rmsnorm_bwd: pointers must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int nparts = ody_rmsnorm_bwd_partials(T);
+  const int rpb = (T + nparts - 1) / nparts;
+  const int nblocks = (T + rpb - 1) / rpb;  // <= nparts; rows of dw_partial beyond nblocks are not written
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(rmsnorm_bwd_kernel<bf16>, dim3(nblocks), dim3(256), 0, st, (const bf16*)x,
+                                  (const bf16*)w, rstd, (const bf16*)dy, (bf16*)dx, dw_partial, T, d, rpb),
+               hipLaunchKernelGGL(rmsnorm_bwd_kernel<float>, dim3(nblocks), dim3(256), 0, st, (const float*)x,
+                                  (const float*)w, rstd, (const float*)dy, (float*)dx, dw_partial, T, d, rpb));
+  int rc = ody_check_launch("rmsnorm_bwd");
+  if (rc || !dw) return rc;
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(colsum_kernel<bf16>, dim3((d + 255) / 256), dim3(256), 0, st, dw_partial, (bf16*)dw,
+                                  nblocks, d),
+               hipLaunchKernelGGL(colsum_kernel<float>, dim3((d + 255) / 256), dim3(256), 0, st, dw_partial,
+                                  (float*)dw, nblocks, d));
+  return ody_check_launch("rmsnorm_bwd_colsum");
+}
+
+extern "C" int ody_rope(void* x, const int64_t* position_ids, const float* inv_freq, int B, int L, int n_rot, int D,
+                        int64_t sx_b, int64_t sx_l, int64_t sx_h, float base, int inverse, int dtype, void* stream) {
+  ODY_REQUIRE(x, ODY_ERR_NULL, "ody_rope: x is NULL");
+  ODY_REQUIRE(B > 0 && L > 0 && n_rot >= 0 && D > 0, ODY_ERR_BAD_SHAPE, "ody_rope: B=%d L=%d n_rot=%d D=%d", B, L,
+              n_rot, D);
+  const int n = dtype == ODY_BF16 ? 8 : 4;
+  ODY_REQUIRE(D % (2 * n) == 0, ODY_ERR_UNSUPPORTED, "ody_rope: D=%d must be a multiple of %d", D, 2 * n);
+  ODY_REQUIRE(ody_aligned16(x) && sx_b % n == 0 && sx_l % n == 0 && sx_h % n == 0, ODY_ERR_MISALIGNED,
+              "ody_rope: x needs a 16-byte aligned pointer and strides that are multiples of %d", n);
+  ODY_REQUIRE(inv_freq || base > 0.f, ODY_ERR_BAD_SHAPE, "ody_rope: base must be positive");
+  if (n_rot == 0) return ODY_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = (int64_t)B * L * (D / 2 / n);
+  const float l2b = inv_freq ? 0.f : log2f(base);
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(rope_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st, (bf16*)x, position_ids,
+                                  inv_freq, B, L, n_rot, D, sx_b, sx_l, sx_h, l2b, inverse),
+               hipLaunchKernelGGL(rope_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st, (float*)x,
+                                  position_ids, inv_freq, B, L, n_rot, D, sx_b, sx_l, sx_h, l2b, inverse));
+  return ody_check_launch("rope");
+}
+
+extern "C" int ody_swiglu_fwd(const void* gate_up, void* h, int T, int I, int64_t ld_gu, int64_t ld_h, int dtype,
+                              void* stream) {
+  ODY_REQUIRE(gate_up && h, ODY_ERR_NULL, "ody_swiglu_fwd: NULL pointer");
+  ODY_REQUIRE(T > 0 && I > 0 && ld_gu >= 2 * (int64_t)I && ld_h >= I, ODY_ERR_BAD_SHAPE,
+              "ody_swiglu_fwd: T=%d I=%d ld_gu=%lld ld_h=%lld", T, I, (long long)ld_gu, (long long)ld_h);
+  const int n = dtype == ODY_BF16 ? 8 : 4;
+  ODY_REQUIRE(I % n == 0, ODY_ERR_UNSUPPORTED, "ody_swiglu_fwd: I=%d must be a multiple of %d", I, n);
+  ODY_REQUIRE(ody_aligned16(gate_up) && ody_aligned16(h) && ld_gu % n == 0 && ld_h % n == 0, ODY_ERR_MISALIGNED,
+              "ody_swiglu_fwd: 16-byte alignment of pointers and row strides required");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = (int64_t)T * (I / n);
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(swiglu_fwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st,
+                                  (const bf16*)gate_up, (bf16*)h, T, I, ld_gu, ld_h),
+               hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st,
+                                  (const float*)gate_up, (float*)h, T, I, ld_gu, ld_h));
+  return ody_check_launch("swiglu_fwd");
+}
+
+extern "C" int ody_swiglu_bwd(const void* gate_up, const void* dh, void* d_gate_up, int T, int I, int64_t ld_gu,
+                              int64_t ld_dh, int64_t ld_dgu, int dtype, void* stream) {
+  ODY_REQUIRE(gate_up && dh && d_gate_up, ODY_ERR_NULL, "ody_swiglu_bwd: NULL pointer");
+  ODY_REQUIRE(T > 0 && I > 0 && ld_gu >= 2 * (int64_t)I && ld_dh >= I && ld_dgu >= 2 * (int64_t)I, ODY_ERR_BAD_SHAPE,
+              "ody_swiglu_bwd: bad sizes T=%d I=%d", T, I);
+  const int n = dtype == ODY_BF16 ? 8 : 4;
+  ODY_REQUIRE(I % n == 0, ODY_ERR_UNSUPPORTED, "ody_swiglu_bwd: I=%d must be a multiple of %d", I, n);
+  ODY_REQUIRE(ody_aligned16(gate_up) && ody_aligned16(dh) && ody_aligned16(d_gate_up) && ld_gu % n == 0 &&
+                  ld_dh % n == 0 && ld_dgu % n == 0,
+              ODY_ERR_MISALIGNED, "ody_swiglu_bwd: 16-byte alignment of pointers and row strides required");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = (int64_t)T * (I / n);
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(swiglu_bwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st,
+                                  (const bf16*)gate_up, (const bf16*)dh, (bf16*)d_gate_up, T, I, ld_gu, ld_dh, ld_dgu),
+               hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st,
+                                  (const float*)gate_up, (const float*)dh, (float*)d_gate_up, T, I, ld_gu, ld_dh,
+                                  ld_dgu));
+  return ody_check_launch("swiglu_bwd");
+}
+
+extern "C" int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk, const float* lse_blk, int B, int L,
+                             int H, int D, int64_t sb_b, int64_t sb_l, int64_t sb_h, int dtype, void* stream) {
+  ODY_REQUIRE(out_acc && lse_acc && out_blk && lse_blk, ODY_ERR_NULL, "ody_lse_merge: NULL pointer");
+  ODY_REQUIRE(B > 0 && L > 0 && H > 0 && D > 0, ODY_ERR_BAD_SHAPE, "ody_lse_merge: B=%d L=%d H=%d D=%d", B, L, H, D);
+  ODY_REQUIRE(D % 4 == 0 && D <= 256 && (64 % (D / 4) == 0), ODY_ERR_UNSUPPORTED,
+              "ody_lse_merge: D=%d must be 4 times a power of two, at most 256", D);
+  ODY_REQUIRE(ody_aligned16(out_acc) && ody_aligned16(out_blk) && sb_b % 4 == 0 && sb_l % 4 == 0 && sb_h % 4 == 0,
+              ODY_ERR_MISALIGNED, "ody_lse_merge: alignment");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t total = (int64_t)B * L * H * (D / 4);
+  ODY_BY_DTYPE(dtype,
+               hipLaunchKernelGGL(lse_merge_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st, out_acc, lse_acc,
+                                  (const bf16*)out_blk, lse_blk, B, L, H, D, sb_b, sb_l, sb_h),
+               hipLaunchKernelGGL(lse_merge_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st, out_acc, lse_acc,
+                                  (const float*)out_blk, lse_blk, B, L, H, D, sb_b, sb_l, sb_h));
+  return ody_check_launch("lse_merge");
+}

@@ -1,0 +1,296 @@
+// Dense linears: C (M, N) = op(A) . op(B) for the three products of a linear
+// layer (forward NT, dgrad NN, wgrad TN).
+//
+// bf16: v_mfma_f32_32x32x16_bf16, 4 wavefronts in a 2 x 2 arrangement, each
+// owning WM x WN accumulator tiles of 32 x 32; operands are staged through LDS
+// in K-slabs of 64, double-buffered, filled with 16-byte global loads issued one
+// slab ahead.  An operand whose memory is contiguous along K is kept as
+// [rows][64 + 8] and read with 16-byte row reads; one that is contiguous along
+// M or N is kept as [64][cols + 32] and read with the LDS transpose read, so no
+// operand is ever transposed in global memory.  The product is computed as
+// C^T = op(B)^T . op(A)^T so that a lane ends up with 4 consecutive N per
+// register quad and writes 8-byte pieces of C rows.
+//
+// fp32: 64 x 64 tiles on the vector ALUs (the fp32 configuration is small and
+// its 1e-4 tolerance rules out bf16 inputs).
+#include "ody_common.h"
+
+namespace {
+
+// ------------------------------------------------------------------ bf16 MFMA
+constexpr int BK = 64;
+
+// Operand tile in LDS.  KC = true: memory is (rows, K) row-major -> [ROWS][BK+8].
+//                       KC = false: memory is (K, rows) row-major -> [BK][ROWS+32].
+template <int ROWS, bool KC>
+struct OperandTile {
+  static constexpr int PITCH = KC ? (BK + 8) : (ROWS + 32);
+  static constexpr int ELEMS = KC ? ROWS * PITCH : BK * PITCH;
+  static constexpr int CHUNKS = ROWS * BK / 8 / 256;  // 16-byte chunks per thread
+  bf16x8 r[CHUNKS];
+
+  // row0: first row (M or N index) of the tile; k0: first K index
+  __device__ __forceinline__ void gload(const bf16* base, int64_t ld, int row0, int k0, int nrows, int K, int tid) {
+#pragma unroll
+    for (int j = 0; j < CHUNKS; j++) {
+      const int c = tid + 256 * j;
+      int rr, kk;
+      if (KC) { rr = c / (BK / 8); kk = (c % (BK / 8)) * 8; }
+      else { kk = c / (ROWS / 8); rr = (c % (ROWS / 8)) * 8; }
+      const int gr = row0 + rr, gk = k0 + kk;
+      bool ok;
+      const bf16* src;
+      if (KC) { ok = gr < nrows && gk < K; src = base + (int64_t)gr * ld + gk; }   // K % 8 == 0: chunk all in or out
+      else { ok = gk < K && gr < nrows; src = base + (int64_t)gk * ld + gr; }      // rows % 8 == 0 likewise
+      r[j] = ok ? *reinterpret_cast<const bf16x8*>(src) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+  __device__ __forceinline__ void sstore(bf16* lds, int tid) const {
+#pragma unroll
+    for (int j = 0; j < CHUNKS; j++) {
+      const int c = tid + 256 * j;
+      int rr, kk;
+      if (KC) { rr = c / (BK / 8); kk = (c % (BK / 8)) * 8; *reinterpret_cast<bf16x8*>(lds + rr * PITCH + kk) = r[j]; }
+      else { kk = c / (ROWS / 8); rr = (c % (ROWS / 8)) * 8; *reinterpret_cast<bf16x8*>(lds + kk * PITCH + rr) = r[j]; }
+    }
+  }
+  // MFMA operand for tile rows [r32, r32+32), k-step ks (16 K values): lane (g, i) gets row r32+i, k = 16ks+8g..+7
+  __device__ static __forceinline__ bf16x8 frag(const bf16* lds, int r32, int ks, int g, int i) {
+    if (KC) {
+      return *reinterpret_cast<const bf16x8*>(lds + (r32 + i) * PITCH + 16 * ks + 8 * g);
+    } else {
+      const bf16* p = lds + (16 * ks + 8 * g + ((i & 15) >> 2)) * PITCH + r32 + 16 * (i >> 4) + 4 * (i & 3);
+      return concat4(lds_read_tr16(p), lds_read_tr16(p + 4 * PITCH));
+    }
+  }
+};
+
+template <int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
+                                                        bf16* __restrict__ C, const bf16* __restrict__ bias, int M,
+                                                        int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                                                        int accumulate, int tiles_m, int tiles_n) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;  // block tile
+  typedef OperandTile<TM, A_KC> TA;
+  typedef OperandTile<TN, B_KC> TB;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* As = reinterpret_cast<bf16*>(smem_raw);  // [2][TA::ELEMS]
+  bf16* Bs = As + 2 * TA::ELEMS;                 // [2][TB::ELEMS]
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // Block -> tile.  Consecutive workgroup ids go round-robin over the 8 XCDs, each
+  // with its own L2: give every XCD a contiguous range of tiles, and inside the
+  // range walk down M in groups so that neighbours share the B panel.
+  int pid = blockIdx.x;
+  const int nblk = tiles_m * tiles_n;
+  if (nblk % 8 == 0) pid = (pid % 8) * (nblk / 8) + pid / 8;
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int gid = pid / per_group, first_m = gid * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int tm = first_m + (pid % per_group) % gsz, tn = (pid % per_group) / gsz;
+  const int m0 = tm * TM, n0 = tn * TN;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int a = 0; a < WM; a++)
+#pragma unroll
+    for (int b = 0; b < WN; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+  TA ta;
+  TB tb;
+  const int nk = (K + BK - 1) / BK;
+  ta.gload(A, lda, m0, 0, M, K, tid);
+  tb.gload(B, ldb, n0, 0, N, K, tid);
+  ta.sstore(As, tid);
+  tb.sstore(Bs, tid);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; kt++) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) {
+      ta.gload(A, lda, m0, (kt + 1) * BK, M, K, tid);
+      tb.gload(B, ldb, n0, (kt + 1) * BK, N, K, tid);
+    }
+    const bf16* Ab = As + buf * TA::ELEMS;
+    const bf16* Bb = Bs + buf * TB::ELEMS;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ks++) {
+      bf16x8 af[WM], bfr[WN];
+#pragma unroll
+      for (int a = 0; a < WM; a++) af[a] = TA::frag(Ab, 32 * (wm * WM + a), ks, g, i);
+#pragma unroll
+      for (int b = 0; b < WN; b++) bfr[b] = TB::frag(Bb, 32 * (wn * WN + b), ks, g, i);
+#pragma unroll
+      for (int a = 0; a < WM; a++)
+#pragma unroll
+        for (int b = 0; b < WN; b++) acc[a][b] = mfma32(bfr[b], af[a], acc[a][b]);  // rows = n, cols = m
+    }
+    if (kt + 1 < nk) {
+      ta.sstore(As + (buf ^ 1) * TA::ELEMS, tid);
+      tb.sstore(Bs + (buf ^ 1) * TB::ELEMS, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane (g, i) holds column m = i, rows n = 8*(r/4) + 4g + r%4
+#pragma unroll
+  for (int a = 0; a < WM; a++) {
+    const int m = m0 + 32 * (wm * WM + a) + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int b = 0; b < WN; b++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + 32 * (wn * WN + b) + 8 * q + 4 * g;
+        if (n >= N) continue;  // N % 8 == 0: a quad is all in or all out
+        bf16* dst = C + (int64_t)m * ldc + n;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+        if (bias) {
+          const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n);
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+        }
+        if (accumulate) {
+          const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)old[e];
+        }
+        bf16x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = (bf16)v[e];
+        *reinterpret_cast<bf16x4*>(dst) = w;
+      }
+    }
+  }
+}
+
+template <int WM, int WN, bool A_KC, bool B_KC>
+int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, int N, int K, int64_t lda, int64_t ldb,
+                int64_t ldc, int accumulate, hipStream_t st) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
+  constexpr size_t smem = 2 * sizeof(bf16) * (OperandTile<TM, A_KC>::ELEMS + OperandTile<TN, B_KC>::ELEMS);
+  static bool attr_set = false;
+  auto kern = &gemm_bf16_kernel<WM, WN, A_KC, B_KC>;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      ody_set_error("ody_gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+      return ODY_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), smem, st, A, B, C, bias, M, N, K, lda, ldb, ldc,
+                     accumulate, tiles_m, tiles_n);
+  return ody_check_launch("gemm_bf16");
+}
+
+template <bool A_KC, bool B_KC>
+int dispatch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, int N, int K, int64_t lda,
+                  int64_t ldb, int64_t ldc, int accumulate, hipStream_t st) {
+  // large problems: 256 x 256 tiles; otherwise 128 x 128 so that the grid still covers the chip
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  if (big_tiles >= 192) return launch_bf16<4, 4, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, st);
+  return launch_bf16<2, 2, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, st);
+}
+
+// ------------------------------------------------------------------ fp32 SIMT
+// A(m, k) = A[m * sam + k * sak], B(k, n) = B[k * sbk + n * sbn]
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
+                                                       float* __restrict__ C, const float* __restrict__ bias, int M,
+                                                       int N, int K, int64_t sam, int64_t sak, int64_t sbk,
+                                                       int64_t sbn, int64_t ldc, int accumulate) {
+  constexpr int T = 64, KB = 16;
+  __shared__ float As[KB][T + 4];
+  __shared__ float Bs[KB][T + 4];
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += KB) {
+    // 64 x 16 elements per operand, 4 per thread; pick the thread->element map that
+    // walks the unit-stride direction of each operand
+    for (int e = tid; e < T * KB; e += 256) {
+      int mm, kk;
+      if (sak == 1) { kk = e % KB; mm = e / KB; } else { mm = e % T; kk = e / T; }
+      const int gm = m0 + mm, gk = k0 + kk;
+      As[kk][mm] = (gm < M && gk < K) ? A[gm * sam + gk * sak] : 0.f;
+      int nn, kb;
+      if (sbk == 1) { kb = e % KB; nn = e / KB; } else { nn = e % T; kb = e / T; }
+      const int gn = n0 + nn, gk2 = k0 + kb;
+      Bs[kb][nn] = (gn < N && gk2 < K) ? B[gk2 * sbk + gn * sbn] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < KB; kk++) {
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) a[u] = As[kk][ty * 4 + u], b[u] = Bs[kk][tx * 4 + u];
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[u][v] = fmaf(a[u], b[v], acc[u][v]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < 4; u++) {
+    const int m = m0 + ty * 4 + u;
+    if (m >= M) continue;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int n = n0 + tx * 4 + v;
+      if (n >= N) continue;
+      float r = acc[u][v];
+      if (bias) r += bias[n];
+      if (accumulate) r += C[(int64_t)m * ldc + n];
+      C[(int64_t)m * ldc + n] = r;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias, int M, int N, int K,
+                        int64_t lda, int64_t ldb, int64_t ldc, int accumulate, int dtype, void* stream) {
+  ODY_REQUIRE(A && B && C, ODY_ERR_NULL, "ody_gemm: NULL pointer");
+  ODY_REQUIRE(M > 0 && N > 0 && K > 0, ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d N=%d K=%d", M, N, K);
+  ODY_REQUIRE(op == ODY_GEMM_NT || op == ODY_GEMM_NN || op == ODY_GEMM_TN, ODY_ERR_UNSUPPORTED, "ody_gemm: op %d", op);
+  const int a_cols = (op == ODY_GEMM_TN) ? M : K, b_cols = (op == ODY_GEMM_NT) ? K : N;
+  ODY_REQUIRE(lda >= a_cols && ldb >= b_cols && ldc >= N, ODY_ERR_BAD_SHAPE,
+              "ody_gemm: leading dimension smaller than the row length (lda=%lld ldb=%lld ldc=%lld)", (long long)lda,
+              (long long)ldb, (long long)ldc);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_F32) {
+    int64_t sam, sak, sbk, sbn;
+    if (op == ODY_GEMM_TN) { sam = 1; sak = lda; } else { sam = lda; sak = 1; }
+    if (op == ODY_GEMM_NT) { sbk = 1; sbn = ldb; } else { sbk = ldb; sbn = 1; }
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    ODY_REQUIRE(grid.y <= 65535, ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d too large for the fp32 path", M);
+    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, st, (const float*)A, (const float*)B, (float*)C,
+                       (const float*)bias, M, N, K, sam, sak, sbk, sbn, ldc, accumulate);
+    return ody_check_launch("gemm_f32");
+  }
+  ODY_REQUIRE(dtype == ODY_BF16, ODY_ERR_UNSUPPORTED, "ody_gemm: dtype %d unknown", dtype);
+  // 16-byte vectors along the contiguous direction of every matrix
+  ODY_REQUIRE(ody_aligned16(A) && ody_aligned16(B) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0) &&
+                  (!bias || (reinterpret_cast<uintptr_t>(bias) & 7u) == 0),
+              ODY_ERR_MISALIGNED, "ody_gemm: A and B must be 16-byte aligned, C and bias 8-byte aligned");
+  ODY_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0, ODY_ERR_MISALIGNED,
+              "ody_gemm: lda and ldb must be multiples of 8, ldc of 4");
+  ODY_REQUIRE(N % 8 == 0 && a_cols % 8 == 0 && b_cols % 8 == 0, ODY_ERR_UNSUPPORTED,
+              "ody_gemm: bf16 path needs N and the contiguous extents of A and B to be multiples of 8 "
+              "(M=%d N=%d K=%d op=%d)", M, N, K, op);
+  const bf16 *a = (const bf16*)A, *b = (const bf16*)B, *bs = (const bf16*)bias;
+  bf16* c = (bf16*)C;
+  if (op == ODY_GEMM_NT) return dispatch_bf16<true, true>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
+  if (op == ODY_GEMM_NN) return dispatch_bf16<true, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
+  return dispatch_bf16<false, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
+}

@@ -1,0 +1,299 @@
+"""Tensor-level wrappers of the C ABI (torch supplies device memory and the
+stream, nothing else) and the autograd functions built from them.
+
+Every function requires CUDA(HIP) tensors and raises otherwise: the HIP library
+is the only compute path.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import GEMM_NN, GEMM_NT, GEMM_TN
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.ODY_BF16
+    if t.dtype == torch.float32:
+        return _lib.ODY_F32
+    raise TypeError(f"odysseus_transformer_amd supports bfloat16 and float32 tensors, got {t.dtype}")
+
+
+def _need_gpu(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "odysseus_transformer_amd ops run only on a HIP device (tensor is on "
+                f"{t.device}); there is no CPU implementation in this package")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _blhd(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
+    if t.dim() != 4:
+        raise ValueError(f"{name} must be (B, L, H, D), got {tuple(t.shape)}")
+    if t.stride(3) != 1:
+        raise ValueError(f"{name}: head_dim must be contiguous (stride {t.stride()})")
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+# --------------------------------------------------------------------------- attention
+def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=None):
+    """q (B, Lq, Hq, D), k/v (B, Lk, Hkv, D) -> out (B, Lq, Hq, D), lse (B, Hq, Lq) fp32."""
+    _need_gpu(q, k, v)
+    B, Lq, Hq, D = q.shape
+    Lk, Hkv = k.shape[1], k.shape[2]
+    if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D:
+        raise ValueError(f"k {tuple(k.shape)} / v {tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if out is None:
+        out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    _lib.call("ody_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+              B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
+              scale, int(causal), _dt(q), _stream())
+    return out, lse
+
+
+def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
+             dq=None, dk=None, dv=None, accumulate_dq: bool = False):
+    """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step."""
+    _need_gpu(q, k, v, out, lse, dout)
+    B, Lq, Hq, D = q.shape
+    Lk, Hkv = k.shape[1], k.shape[2]
+    if dq is None:
+        if accumulate_dq:
+            raise ValueError("accumulate_dq needs an existing dq")
+        dq = torch.empty_like(q)
+    dk = torch.empty_like(k) if dk is None else dk
+    dv = torch.empty_like(v) if dv is None else dv
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    lib = _lib.load()
+    ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Hq)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
+    _lib.call("ody_attn_bwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+              dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+              B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
+              *_blhd(dout, "dout"), *_blhd(dq, "dq"), *_blhd(dk, "dk"), *_blhd(dv, "dv"),
+              scale, int(causal), int(accumulate_dq), _dt(q), ws.data_ptr(), ws_bytes, _stream())
+    return dq, dk, dv
+
+
+def lse_merge_(out_acc, lse_acc, out_blk, lse_blk) -> None:
+    """In place: folds (out_blk, lse_blk) into the fp32 running (out_acc, lse_acc)."""
+    _need_gpu(out_acc, lse_acc, out_blk, lse_blk)
+    B, L, H, D = out_blk.shape
+    if out_acc.dtype != torch.float32 or not out_acc.is_contiguous() or tuple(out_acc.shape) != (B, L, H, D):
+        raise ValueError("out_acc must be a contiguous float32 (B, L, H, D) tensor")
+    for t, n in ((lse_acc, "lse_acc"), (lse_blk, "lse_blk")):
+        if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (B, H, L):
+            raise ValueError(f"{n} must be a contiguous float32 (B, H, L) tensor")
+    _lib.call("ody_lse_merge", out_acc.data_ptr(), lse_acc.data_ptr(), out_blk.data_ptr(), lse_blk.data_ptr(),
+              B, L, H, D, *_blhd(out_blk, "out_blk"), _dt(out_blk), _stream())
+
+
+# --------------------------------------------------------------------------- linears
+def _rowmajor2d(t: torch.Tensor, name: str) -> int:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be 2-D with unit column stride, got shape {tuple(t.shape)} stride {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def gemm(op: int, a, b, bias=None, out=None, accumulate: bool = False):
+    """op NT: a (M,K) b (N,K); NN: a (M,K) b (K,N); TN: a (K,M) b (K,N) -> (M,N)."""
+    _need_gpu(a, b, bias, out)
+    if op == GEMM_NT:
+        (M, K), (N, K2) = a.shape, b.shape
+    elif op == GEMM_NN:
+        (M, K), (K2, N) = a.shape, b.shape
+    elif op == GEMM_TN:
+        (K, M), (K2, N) = a.shape, b.shape
+    else:
+        raise ValueError(f"unknown gemm op {op}")
+    if K != K2:
+        raise ValueError(f"inner dimensions differ: {tuple(a.shape)} vs {tuple(b.shape)} for op {op}")
+    if a.dtype != b.dtype:
+        raise TypeError(f"dtype mismatch {a.dtype} vs {b.dtype}")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an existing out")
+        out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    _lib.call("ody_gemm", op, a.data_ptr(), b.data_ptr(), out.data_ptr(), 0 if bias is None else bias.data_ptr(),
+              M, N, K, _rowmajor2d(a, "a"), _rowmajor2d(b, "b"), _rowmajor2d(out, "out"),
+              int(accumulate), _dt(a), _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- elementwise
+def swiglu_fwd(gate_up):
+    _need_gpu(gate_up)
+    gu = gate_up.reshape(-1, gate_up.shape[-1])
+    T, I2 = gu.shape
+    h = torch.empty((T, I2 // 2), dtype=gu.dtype, device=gu.device)
+    _lib.call("ody_swiglu_fwd", gu.data_ptr(), h.data_ptr(), T, I2 // 2, _rowmajor2d(gu, "gate_up"), h.stride(0),
+              _dt(gu), _stream())
+    return h.view(*gate_up.shape[:-1], I2 // 2)
+
+
+def swiglu_bwd(gate_up, dh):
+    _need_gpu(gate_up, dh)
+    gu = gate_up.reshape(-1, gate_up.shape[-1])
+    d = dh.reshape(-1, dh.shape[-1])
+    if d.stride(1) != 1:
+        d = d.contiguous()
+    T, I2 = gu.shape
+    dgu = torch.empty((T, I2), dtype=gu.dtype, device=gu.device)
+    _lib.call("ody_swiglu_bwd", gu.data_ptr(), d.data_ptr(), dgu.data_ptr(), T, I2 // 2,
+              _rowmajor2d(gu, "gate_up"), _rowmajor2d(d, "dh"), dgu.stride(0), _dt(gu), _stream())
+    return dgu.view(gate_up.shape)
+
+
+def rmsnorm_fwd(x, weight, eps: float = 1e-6):
+    _need_gpu(x, weight)
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    T, d = x2.shape
+    y = torch.empty_like(x2)
+    rstd = torch.empty(T, dtype=torch.float32, device=x.device)
+    _lib.call("ody_rmsnorm_fwd", x2.data_ptr(), weight.data_ptr(), y.data_ptr(), rstd.data_ptr(), T, d, float(eps),
+              _dt(x2), _stream())
+    return y.view(x.shape), rstd
+
+
+def rmsnorm_bwd(x, weight, rstd, dy):
+    _need_gpu(x, weight, rstd, dy)
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+    T, d = x2.shape
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(weight)
+    nparts = _lib.load().ody_rmsnorm_bwd_partials(T)
+    partial = torch.empty((nparts, d), dtype=torch.float32, device=x.device)
+    _lib.call("ody_rmsnorm_bwd", x2.data_ptr(), weight.data_ptr(), rstd.data_ptr(), dy2.data_ptr(), dx.data_ptr(),
+              partial.data_ptr(), dw.data_ptr(), T, d, _dt(x2), _stream())
+    return dx.view(x.shape), dw
+
+
+_INV_FREQ_CACHE = {}
+
+
+def rope_inv_freq(head_dim: int, base: float, device) -> torch.Tensor:
+    """base^(-2j/D), evaluated on the host in fp32 the way HF's rotary module does, then moved."""
+    key = (head_dim, float(base), str(device))
+    t = _INV_FREQ_CACHE.get(key)
+    if t is None:
+        t = (1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))).to(device)
+        _INV_FREQ_CACHE[key] = t
+    return t
+
+
+def rope_(x, n_rot: int, position_ids=None, base: float = 10000.0, inverse: bool = False, inv_freq=None) -> None:
+    """Rotates heads [0, n_rot) of x (B, L, H, D) in place."""
+    _need_gpu(x, position_ids, inv_freq)
+    B, L, H, D = x.shape
+    if n_rot > H:
+        raise ValueError(f"n_rot={n_rot} exceeds the {H} heads of x")
+    if inv_freq is None:
+        inv_freq = rope_inv_freq(D, base, x.device)
+    pos_ptr = 0
+    if position_ids is not None:
+        position_ids = position_ids.to(torch.int64).expand(B, L).contiguous()
+        pos_ptr = position_ids.data_ptr()
+    _lib.call("ody_rope", x.data_ptr(), pos_ptr, inv_freq.data_ptr(), B, L, n_rot, D, *_blhd(x, "x"),
+              float(base), int(inverse), _dt(x), _stream())
+
+
+# --------------------------------------------------------------------------- autograd
+class FlashAttnFunc(torch.autograd.Function):
+    """Causal/full attention with GQA over (B, L, H, D) tensors; returns (out, lse)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, softmax_scale, causal):
+        out, lse = attn_fwd(q, k, v, causal=causal, scale=softmax_scale)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.softmax_scale, ctx.causal = softmax_scale, causal
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, k, v, out, lse = ctx.saved_tensors
+        if dout.stride(3) != 1:
+            dout = dout.contiguous()
+        dq, dk, dv = attn_bwd(q, k, v, out, lse, dout, causal=ctx.causal, scale=ctx.softmax_scale)
+        return dq, dk, dv, None, None
+
+
+def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[float] = None, causal: bool = False,
+                    return_lse: bool = False):
+    """Signature of the routine the reference reaches at decoder/odysseus.py:256-263.
+
+    Dropout is not implemented (the training loop of the reference runs with
+    attention_dropout = 0.0); a non-zero value raises."""
+    if dropout_p != 0.0:
+        raise NotImplementedError("attention dropout is not implemented (the reference runs with 0.0)")
+    out, lse = FlashAttnFunc.apply(q, k, v, softmax_scale, causal)
+    return (out, lse) if return_lse else out
+
+
+class RMSNormFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        y, rstd = rmsnorm_fwd(x, weight, eps)
+        ctx.save_for_backward(x, weight, rstd)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, rstd = ctx.saved_tensors
+        dx, dw = rmsnorm_bwd(x, weight, rstd, dy)
+        return dx, dw, None
+
+
+class SwiGLUFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, gate_up):
+        ctx.save_for_backward(gate_up)
+        return swiglu_fwd(gate_up)
+
+    @staticmethod
+    def backward(ctx, dh):
+        (gate_up,) = ctx.saved_tensors
+        return swiglu_bwd(gate_up, dh)
+
+
+class RoPEFunc(torch.autograd.Function):
+    """Rotates the first n_rot heads of a packed (B, L, H, D) projection; out of place for autograd."""
+
+    @staticmethod
+    def forward(ctx, x, n_rot, position_ids, base):
+        y = x.clone()
+        rope_(y, n_rot, position_ids, base)
+        ctx.n_rot, ctx.base = n_rot, base
+        ctx.position_ids = position_ids
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        dx = dy.clone() if dy.stride(3) == 1 else dy.contiguous()
+        rope_(dx, ctx.n_rot, ctx.position_ids, ctx.base, inverse=True)
+        return dx, None, None, None
+
+
+def rmsnorm(x, weight, eps: float = 1e-6):
+    return RMSNormFunc.apply(x, weight, eps)
+
+
+def swiglu(gate_up):
+    return SwiGLUFunc.apply(gate_up)
+
+
+def apply_rope_packed(qkv, n_rot: int, position_ids=None, base: float = 10000.0):
+    return RoPEFunc.apply(qkv, n_rot, position_ids, base)
