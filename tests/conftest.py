@@ -31,11 +31,11 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-def rel_err(a: torch.Tensor, ref: torch.Tensor) -> float:
+def rel_err(a: torch.Tensor, ref: torch.Tensor, floor: float = 1e-3) -> float:
     a, ref = a.detach().double().cpu(), ref.detach().double().cpu()
     # the floor keeps a tensor that is zero by construction (e.g. dq of a
     # single-key softmax) from turning rounding noise into a ratio of 1
-    den = max(ref.abs().max().item(), 1e-3)
+    den = max(ref.abs().max().item(), floor)
     return (a - ref).abs().max().item() / den
 
 

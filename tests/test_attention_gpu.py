@@ -49,8 +49,10 @@ def test_attention_fwd_bwd(case, dtype, dev):
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
     dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal)
     torch.cuda.synchronize()
-    assert rel_err(dq, dq_ref) <= tol, "dq"
-    assert rel_err(dk, dk_ref) <= tol, "dk"
+    # with a single key dS = P (dP - delta) is identically zero: compare on the scale of the inputs
+    floor = 1.0 if Lk == 1 else 1e-3
+    assert rel_err(dq, dq_ref, floor) <= tol, "dq"
+    assert rel_err(dk, dk_ref, floor) <= tol, "dk"
     assert rel_err(dv, dv_ref) <= tol, "dv"
 
 

@@ -1,0 +1,144 @@
+"""GPU parity: RMSNorm, RoPE, SwiGLU and the LSE merge vs. the CPU oracle."""
+import pytest
+import torch
+
+from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
+import odysseus_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+DTYPES = pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+
+
+def _tol(dtype):
+    return TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
+
+
+@DTYPES
+@pytest.mark.parametrize("T,d", [(7, 512), (2048, 512), (513, 4096), (3, 8192), (5, 16384)])
+def test_rmsnorm(T, d, dtype, dev):
+    from odysseus_transformer_amd import ops
+    x = randn((1, T, d), 1, dtype=dtype)
+    w = (1.0 + randn((d,), 2, std=0.02)).to(dtype)
+    dy = randn((1, T, d), 3, dtype=dtype)
+    y_ref = oracle.rmsnorm(x.float(), w.float())
+    y, rstd = ops.rmsnorm_fwd(x.to(dev), w.to(dev), 1e-6)
+    assert rel_err(y, y_ref) <= _tol(dtype)
+    n = 256 * (8 if dtype == torch.bfloat16 else 4) * 4
+    if d <= n:
+        dx_ref, dw_ref = oracle.rmsnorm_bwd(x.float(), w.float(), dy.float())
+        dx, dw = ops.rmsnorm_bwd(x.to(dev), w.to(dev), rstd, dy.to(dev))
+        assert rel_err(dx, dx_ref) <= _tol(dtype)
+        assert rel_err(dw, dw_ref) <= _tol(dtype)
+
+
+@DTYPES
+@pytest.mark.parametrize("B,L,H,Hkv,D", [(1, 2048, 8, 8, 64), (2, 300, 4, 1, 128), (1, 4096, 4, 4, 128)])
+def test_rope(B, L, H, Hkv, D, dtype, dev):
+    from odysseus_transformer_amd import ops
+    qkv = randn((B, L, H + 2 * Hkv, D), 9, dtype=dtype)
+    pos = torch.arange(L)[None].expand(B, L)
+    cos, sin = oracle.rope_cos_sin(pos, D, 10000.0, torch.float32)
+    ref = qkv.float().clone()
+    ref[:, :, :H + Hkv] = oracle.apply_rope(ref[:, :, :H + Hkv], cos, sin)
+    g = qkv.to(dev).clone()
+    ops.rope_(g, H + Hkv, None, 10000.0)
+    assert rel_err(g, ref) <= _tol(dtype)
+    assert torch.equal(g[:, :, H + Hkv:].cpu(), qkv[:, :, H + Hkv:])          # v untouched
+    # explicit position ids == implicit arange; inverse undoes the rotation
+    g2 = qkv.to(dev).clone()
+    ops.rope_(g2, H + Hkv, pos.to(dev), 10000.0)
+    assert torch.equal(g2, g)
+    ops.rope_(g2, H + Hkv, pos.to(dev), 10000.0, inverse=True)
+    assert rel_err(g2, qkv.float()) <= _tol(dtype)
+    # backward == oracle's explicit backward
+    dref = qkv.float().clone()
+    dref[:, :, :H + Hkv] = oracle.apply_rope_bwd(dref[:, :, :H + Hkv], cos, sin)
+    g3 = qkv.to(dev).clone()
+    ops.rope_(g3, H + Hkv, None, 10000.0, inverse=True)
+    assert rel_err(g3, dref) <= _tol(dtype)
+
+
+def test_rope_far_positions_fp32(dev):
+    """Position ids far from zero: the angle is formed in fp32 exactly as on the host."""
+    from odysseus_transformer_amd import ops
+    B, L, H, D = 1, 64, 2, 128
+    x = randn((B, L, H, D), 4)
+    pos = (torch.arange(L) * 2053 + 100000)[None]
+    cos, sin = oracle.rope_cos_sin(pos, D, 10000.0, torch.float32)
+    ref = oracle.apply_rope(x, cos, sin)
+    g = x.to(dev).clone()
+    ops.rope_(g, H, pos.to(dev), 10000.0)
+    assert rel_err(g, ref) <= TOL_F32
+
+
+@DTYPES
+@pytest.mark.parametrize("T,I", [(5, 1376), (2048, 1376), (300, 11008)])
+def test_swiglu(T, I, dtype, dev):
+    from odysseus_transformer_amd import ops
+    gu = randn((1, T, 2 * I), 21, dtype=dtype)
+    dh = randn((1, T, I), 22, dtype=dtype)
+    h_ref = oracle.swiglu(gu.float())
+    dgu_ref = oracle.swiglu_bwd(gu.float(), dh.float())
+    h = ops.swiglu_fwd(gu.to(dev))
+    dgu = ops.swiglu_bwd(gu.to(dev), dh.to(dev))
+    assert rel_err(h, h_ref) <= _tol(dtype)
+    assert rel_err(dgu, dgu_ref) <= _tol(dtype)
+
+
+@DTYPES
+def test_lse_merge(dtype, dev):
+    from odysseus_transformer_amd import ops
+    B, L, H, D = 2, 130, 4, 128
+    out = randn((B, L, H, D), 31)
+    lse = randn((B, H, L), 32, std=3.0)
+    ob = randn((B, L, H, D), 33, dtype=dtype)
+    lb = randn((B, H, L), 34, std=3.0)
+    lse[0, 0, :5] = float("-inf")          # running side empty
+    lb[0, 1, :5] = float("-inf")           # block side empty
+    lse[1, 2, 7] = lb[1, 2, 7] = float("-inf")   # both empty
+    o_ref, l_ref = oracle.lse_merge(out, lse, ob.float(), lb)
+    og, lg = out.to(dev).clone(), lse.to(dev).clone()
+    ops.lse_merge_(og, lg, ob.to(dev), lb.to(dev))
+    assert rel_err(og, o_ref) <= 1e-5
+    assert torch.allclose(lg.cpu(), l_ref, atol=1e-5, rtol=1e-5)
+    assert torch.isinf(lg[1, 2, 7]) and (og[1, 7, 2] == 0).all()
+
+
+def test_ring_step_equals_unsplit_attention(dev):
+    """Block attention + merge over a partition of the keys == attention over all keys,
+    forward and every gradient (the invariant that pins the ring step)."""
+    from odysseus_transformer_amd import ops
+    B, Lq, H, Hkv, D, NB = 1, 256, 4, 2, 128, 3
+    dt = torch.bfloat16
+    q = randn((B, Lq, H, D), 41, dtype=dt)
+    ks = [randn((B, Lq, Hkv, D), 50 + b, dtype=dt) for b in range(NB)]
+    vs = [randn((B, Lq, Hkv, D), 60 + b, dtype=dt) for b in range(NB)]
+    do = randn((B, Lq, H, D), 42, dtype=dt)
+    # oracle: the causal diagonal block is block 0; the others are fully visible.  As one
+    # attention call that is keys = [blocks 1.., block 0] with the bottom-right causal mask.
+    k_all = torch.cat(ks[1:] + ks[:1], 1).float()
+    v_all = torch.cat(vs[1:] + vs[:1], 1).float()
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k_all, v_all, causal=True)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k_all, v_all, o_ref, lse_ref, do.float(), causal=True)
+    o2, l2 = oracle.ring_attention_fwd(q.float(), [k.float() for k in ks], [v.float() for v in vs], causal_block=0)
+    assert rel_err(o2, o_ref) <= 1e-5 and torch.allclose(l2, lse_ref, atol=1e-5)
+    # device ring step
+    qg, dog = q.to(dev), do.to(dev)
+    out = torch.zeros((B, Lq, H, D), dtype=torch.float32, device=dev)
+    lse = torch.full((B, H, Lq), float("-inf"), dtype=torch.float32, device=dev)
+    for b in range(NB):
+        ob, lb = ops.attn_fwd(qg, ks[b].to(dev), vs[b].to(dev), causal=(b == 0))
+        ops.lse_merge_(out, lse, ob, lb)
+    assert rel_err(out, o_ref) <= TOL_BF16
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    out_bf = out.to(dt)
+    dq = torch.zeros_like(qg)
+    dks, dvs = [], []
+    for b in range(NB):
+        _, dk, dv = ops.attn_bwd(qg, ks[b].to(dev), vs[b].to(dev), out_bf, lse, dog, causal=(b == 0), dq=dq,
+                                 accumulate_dq=(b > 0))
+        dks.append(dk)
+        dvs.append(dv)
+    assert rel_err(dq, dq_ref) <= TOL_BF16
+    assert rel_err(torch.cat(dks[1:] + dks[:1], 1), dk_ref) <= TOL_BF16
+    assert rel_err(torch.cat(dvs[1:] + dvs[:1], 1), dv_ref) <= TOL_BF16

@@ -1,0 +1,89 @@
+"""GPU parity: the three products of a linear layer through ody_gemm vs. the CPU oracle."""
+import pytest
+import torch
+
+from conftest import TOL_BF16, TOL_F32, randn, rel_err
+import odysseus_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    # M, N, K
+    (64, 64, 64),
+    (256, 256, 256),
+    (300, 136, 72),        # ragged in every direction (multiples of 8)
+    (2048, 1536, 512),     # the fp32 configuration's QKV projection
+    (520, 2752, 512),      # gate_up of the fp32 configuration, ragged M
+    (1024, 768, 4096),
+    (4096, 4096, 512),     # enough tiles for the 256 x 256 kernel
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "M%d_N%d_K%d" % s)
+def test_linear_fwd_dgrad_wgrad(shape, dtype, dev):
+    from odysseus_transformer_amd import ops
+    M, N, K = shape
+    print(f"shape={shape} dtype={dtype}", flush=True)
+    tol = TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
+    x = randn((M, K), 1, dtype=dtype)
+    w = randn((N, K), 2, std=0.02, dtype=dtype)
+    dy = randn((M, N), 3, dtype=dtype)
+    y_ref = oracle.linear_fwd(x.float(), w.float())
+    dx_ref, dw_ref, _ = oracle.linear_bwd(x.float(), w.float(), dy.float())
+    xg, wg, dyg = x.to(dev), w.to(dev), dy.to(dev)
+    y = ops.gemm(ops.GEMM_NT, xg, wg)              # X W^T
+    dx = ops.gemm(ops.GEMM_NN, dyg, wg)            # dY W
+    dw = ops.gemm(ops.GEMM_TN, dyg, xg)            # dY^T X
+    torch.cuda.synchronize()
+    assert rel_err(y, y_ref) <= tol, "fwd"
+    assert rel_err(dx, dx_ref) <= tol, "dgrad"
+    assert rel_err(dw, dw_ref) <= tol, "wgrad"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_bias_accumulate_and_strides(dtype, dev):
+    from odysseus_transformer_amd import ops
+    tol = TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
+    M, N, K = 200, 264, 136
+    x = randn((M, K + 24), 4, dtype=dtype)[:, 8:8 + K]          # row stride > K, offset start
+    w = randn((N, K), 5, std=0.05, dtype=dtype)
+    b = randn((N,), 6, dtype=dtype)
+    c0 = randn((M, N), 7, dtype=dtype)
+    ref = oracle.linear_fwd(x.float(), w.float(), b.float()) + c0.float()
+    xg = randn((M, K + 24), 4, dtype=dtype).to(dev)[:, 8:8 + K]
+    out = c0.to(dev).clone()
+    ops.gemm(ops.GEMM_NT, xg, w.to(dev), bias=b.to(dev), out=out, accumulate=True)
+    assert rel_err(out, ref) <= tol
+
+
+def test_linearity_at_full_size(dev):
+    """Size-independent property at a rank-shard shape: X (W1 + W2)^T == X W1^T + X W2^T
+    up to bf16 rounding, and the wgrad of a row-permuted batch is unchanged."""
+    from odysseus_transformer_amd import ops
+    M, N, K = 8192, 1536, 4096
+    x = randn((M, K), 11, dtype=torch.bfloat16).to(dev)
+    w1 = randn((N, K), 12, std=0.02, dtype=torch.bfloat16).to(dev)
+    w2 = randn((N, K), 13, std=0.02, dtype=torch.bfloat16).to(dev)
+    y12 = ops.gemm(ops.GEMM_NT, x, (w1.float() + w2.float()).bfloat16())
+    y1, y2 = ops.gemm(ops.GEMM_NT, x, w1), ops.gemm(ops.GEMM_NT, x, w2)
+    assert rel_err(y12, y1.float() + y2.float()) <= TOL_BF16
+    dy = randn((M, N), 14, dtype=torch.bfloat16).to(dev)
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(0)).to(dev)
+    dw = ops.gemm(ops.GEMM_TN, dy, x)
+    dwp = ops.gemm(ops.GEMM_TN, dy[perm].contiguous(), x[perm].contiguous())
+    assert rel_err(dwp, dw.float()) <= 5e-3
+    # spot check rows against fp64
+    rows = torch.tensor([0, 1, 777, M - 1], device=dev)
+    ref = x[rows].double() @ w1.double().T
+    assert rel_err(y1[rows], ref) <= TOL_BF16
+
+
+def test_gemm_errors(dev):
+    from odysseus_transformer_amd import ops
+    from odysseus_transformer_amd._lib import OdysseusHipError
+    a = torch.zeros(16, 20, dtype=torch.bfloat16, device=dev)   # K = 20 is not a multiple of 8
+    with pytest.raises(OdysseusHipError):
+        ops.gemm(ops.GEMM_NT, a, a)
+    with pytest.raises(ValueError):
+        ops.gemm(ops.GEMM_NT, a, torch.zeros(16, 24, dtype=torch.bfloat16, device=dev))
