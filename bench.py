@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank Odysseus hot path on one MI355X.
+
+A "step" is one causal attention forward + backward over one rank's share of a
+Llama-2-7B layer: 4 heads x 128, L = 32768, bf16, batch 1 (synthetic N(0,1)
+inputs, already resident in HBM).  `value` is the algorithmic TFLOP/s of that step
+(3.5 * 4 * L^2 * D * H / 2 FLOPs).  The same JSON line carries:
+
+  roofline      the dominant kernel's algorithmic FLOP rate against the bf16 dense
+                MFMA peak, its duration measured with HIP events on the launch stream
+  kernels       the same for every attention kernel of the step
+  layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs,
+                RoPE, RMSNorm, SwiGLU) and the resulting tokens/s
+  cpu_baseline  the CPU oracle timed on this host's cores on a bounded sample
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-layer]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+
+# the rank shard the metric is quoted on
+L, H, HKV, D = 32768, 4, 4, 128
+D_MODEL, I_MLP, T_MLP = 4096, 11008, 4096
+
+
+def attn_flops(Lq, Lk, h, d, causal=True):
+    fwd = 4.0 * Lq * Lk * d * h * (0.5 if causal else 1.0)
+    return fwd, 2.5 * fwd
+
+
+def time_gpu(fn, iters, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters
+
+
+def cpu_baseline():
+    """The oracle (plain PyTorch, fp32) on the host cores: causal attention fwd+bwd at
+    4 heads x 128, L = 8192 -- 1/16 of the FLOPs of one benchmark step."""
+    import torch
+    sys.path.insert(0, str(ROOT / "oracle"))
+    import odysseus_oracle as oracle
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    Ls = 8192
+    g = torch.Generator().manual_seed(2000)
+    q, k, v, do = (torch.randn(1, Ls, H, D, generator=g) for _ in range(4))
+    t0 = time.perf_counter()
+    o, lse = oracle.attention_fwd(q, k, v, causal=True)
+    oracle.attention_bwd(q, k, v, o, lse, do, causal=True)
+    dt = time.perf_counter() - t0
+    f, b = attn_flops(Ls, Ls, H, D)
+    return {"value": (f + b) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"causal attention fwd+bwd, {H} heads x {D}, L={Ls} (1/16 of the step's FLOPs), fp32, "
+                      f"{dt:.2f} s wall"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-layer", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU's share of the layer on ONE GPU; collectives and multi-GPU runs are "
+              "not part of this build (--gpus must be 1).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from odysseus_transformer_amd import _lib, ops
+    _lib.load()
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    prop = torch.cuda.get_device_properties(0)
+    dt = torch.bfloat16
+
+    def rn(shape, seed, std=1.0):
+        g = torch.Generator().manual_seed(seed)
+        return (torch.randn(shape, generator=g) * std).to(dt).to(dev)
+
+    # ---- the step: attention fwd + bwd on q/k/v slices of a packed projection buffer
+    qkv = rn((1, L, H + 2 * HKV, D), 2001)
+    q, k, v = qkv[:, :, :H], qkv[:, :, H:H + HKV], qkv[:, :, H + HKV:]
+    do = rn((1, L, H, D), 2002)
+    dqkv = torch.empty_like(qkv)
+    state = {}
+
+    def step():
+        o, lse = ops.attn_fwd(q, k, v, causal=True)
+        ops.attn_bwd(q, k, v, o, lse, do, causal=True, dq=dqkv[:, :, :H], dk=dqkv[:, :, H:H + HKV],
+                     dv=dqkv[:, :, H + HKV:])
+        state["o"] = o
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    _lib.profile_collect()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / a.steps
+    prof = _lib.profile_collect()
+    _lib.profile_enable(False)
+
+    f_fwd, f_bwd = attn_flops(L, L, H, D)
+    # algorithmic FLOPs per launch: the backward's 5 tile products are S, dP, dV, dK (in the
+    # dK/dV kernel) and dQ (in the dQ kernel); the S and dP the dQ kernel recomputes are not counted
+    algo = {"attn_fwd_mfma": f_fwd, "attn_bwd_dkdv": f_bwd * 4 / 5, "attn_bwd_dq": f_bwd * 1 / 5}
+    kernels = {}
+    for name, (n, total_ms, min_ms) in prof.items():
+        avg = total_ms / n
+        kernels[name] = {"launches": n, "avg_ms": round(avg, 4), "min_ms": round(min_ms, 4)}
+        if name in algo:
+            kernels[name]["tflops"] = round(algo[name] / (avg * 1e-3) / 1e12, 1)
+    dom = max(algo, key=lambda n: prof[n][1] / prof[n][0])
+    dom_avg = prof[dom][1] / prof[dom][0]
+    achieved = algo[dom] / (dom_avg * 1e-3) / 1e12
+    traffic = None
+    tf = ROOT / "profiles" / "attn_hbm_traffic.json"
+    if tf.exists():
+        traffic = json.loads(tf.read_text()).get(dom)
+    value = (f_fwd + f_bwd) / sec / 1e12
+
+    out = {
+        "metric": "attention fwd+bwd TFLOP/s (% bf16 MFMA peak) + decoder-layer tokens/s, 1 GPU",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "causal attention fwd+bwd, Llama-2-7B rank shard at N=8: 4 heads x 128, L=32768, "
+                               "batch 1 (BASELINE.json configs[1], attention part)",
+                   "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd},
+        "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+        "device": {"name": prop.name, "cus": prop.multi_processor_count,
+                   "clock_mhz": getattr(prop, "clock_rate", 0) / 1000.0},
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                     "avg_ms": round(dom_avg, 4), "algorithmic_flops_per_launch": algo[dom]},
+        "kernels": kernels,
+    }
+
+    if not a.no_layer:
+        out["layer"] = layer_share(ops, rn, dev, sec)
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+def layer_share(ops, rn, dev, attn_sec):
+    """Times the rest of the rank's share of the layer: the TP-split QKV / O linears over
+    the gathered 32768 tokens, RoPE, and the sequence shard's RMSNorm + SwiGLU MLP over
+    4096 tokens, each forward and backward (fwd, dgrad, wgrad)."""
+    import torch
+    res = {}
+
+    def gemm3(tag, M, N, K):
+        x, w, dy = rn((M, K), 1), rn((N, K), 2, 0.02), rn((M, N), 3)
+        tf = time_gpu(lambda: ops.gemm(ops.GEMM_NT, x, w), 5, 2)
+        td = time_gpu(lambda: ops.gemm(ops.GEMM_NN, dy, w), 5, 2)
+        tw = time_gpu(lambda: ops.gemm(ops.GEMM_TN, dy, x), 5, 2)
+        fl = 2.0 * M * N * K
+        res[tag] = {"M": M, "N": N, "K": K, "fwd_ms": round(tf * 1e3, 3), "dgrad_ms": round(td * 1e3, 3),
+                    "wgrad_ms": round(tw * 1e3, 3),
+                    "tflops": [round(fl / t / 1e12, 1) for t in (tf, td, tw)]}
+        del x, w, dy
+        return tf + td + tw
+
+    def membound(tag, fn, nbytes):
+        t = time_gpu(fn, 10, 3)
+        res[tag] = {"ms": round(t * 1e3, 4), "algorithmic_GBs": round(nbytes / t / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 3)}
+        return t
+
+    t_attn_half = attn_sec
+    t_attn_half += gemm3("qkv_proj", L, (H + 2 * HKV) * D, D_MODEL)
+    t_attn_half += gemm3("o_proj", L, D_MODEL, H * D)
+    qkv = rn((1, L, H + 2 * HKV, D), 5)
+    e = 2
+    rope_bytes = 2 * L * (H + HKV) * D * e
+    t_attn_half += 2 * membound("rope", lambda: ops.rope_(qkv, H + HKV), rope_bytes)
+    del qkv
+
+    t_mlp_half = gemm3("gate_up_proj", T_MLP, 2 * I_MLP, D_MODEL)
+    t_mlp_half += gemm3("down_proj", T_MLP, D_MODEL, I_MLP)
+    gu, dh = rn((T_MLP, 2 * I_MLP), 6), rn((T_MLP, I_MLP), 7)
+    t_mlp_half += membound("swiglu_fwd", lambda: ops.swiglu_fwd(gu), 3 * T_MLP * I_MLP * e)
+    t_mlp_half += membound("swiglu_bwd", lambda: ops.swiglu_bwd(gu, dh), 5 * T_MLP * I_MLP * e)
+    del gu, dh
+    x, w, dy = rn((T_MLP, D_MODEL), 8), rn((D_MODEL,), 9), rn((T_MLP, D_MODEL), 10)
+    _, rstd = ops.rmsnorm_fwd(x, w)
+    t_n = membound("rmsnorm_fwd", lambda: ops.rmsnorm_fwd(x, w), 2 * T_MLP * D_MODEL * e)
+    t_n += membound("rmsnorm_bwd", lambda: ops.rmsnorm_bwd(x, w, rstd, dy), 3 * T_MLP * D_MODEL * e)
+    t_mlp_half += 2 * t_n  # both norms of the layer act on the sequence shard
+    res["attn_half_ms"] = round(t_attn_half * 1e3, 3)
+    res["mlp_half_ms"] = round(t_mlp_half * 1e3, 3)
+    res["attn_half_tokens_per_s"] = round(L / t_attn_half, 1)
+    res["mlp_half_tokens_per_s"] = round(T_MLP / t_mlp_half, 1)
+    # one rank advances its 4096-token shard of the 32768-token layer in attn_half + mlp_half
+    res["layer_tokens_per_s_per_gpu"] = round(T_MLP / (t_attn_half + t_mlp_half), 1)
+    return res
+
+
+if __name__ == "__main__":
+    main()

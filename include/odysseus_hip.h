@@ -44,6 +44,16 @@ enum ody_status {
 const char* ody_last_error(void);
 int ody_version(void);
 
+/* Per-kernel timer (no counterpart in the reference, whose only clock is time.time()
+ * around whole steps, train.py:185-229).  While enabled, every kernel launch of the
+ * library is bracketed by a pair of HIP events on its launch stream.
+ * ody_profile_collect waits for the recorded events, writes one text line per kernel
+ * name -- "name launches total_ms min_ms" -- into out (NUL-terminated, at most cap
+ * bytes) and forgets them.
+ */
+int ody_profile_enable(int on);
+int ody_profile_collect(char* out, size_t cap);
+
 /* ---- attention ---------------------------------------------------------
  * Replaces flash_attn_func(q, k, v, dropout_p=0, softmax_scale, causal) as
  * reached from decoder/odysseus.py:256-263 (via HF _flash_attention_forward),

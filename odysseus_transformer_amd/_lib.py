@@ -20,6 +20,8 @@ _i, _i64, _f, _p, _sz = C.c_int, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
 SIGNATURES = {
     "ody_last_error": (C.c_char_p, []),
     "ody_version": (_i, []),
+    "ody_profile_enable": (_i, [_i]),
+    "ody_profile_collect": (_i, [C.c_char_p, _sz]),
     "ody_attn_fwd": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p]),
     "ody_attn_bwd_workspace_bytes": (_sz, [_i, _i, _i]),
     "ody_attn_bwd": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p]),
@@ -68,3 +70,18 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise OdysseusHipError(name, rc, lib.ody_last_error().decode("utf-8", "replace"))
+
+
+def profile_enable(on: bool) -> None:
+    call("ody_profile_enable", int(on))
+
+
+def profile_collect() -> dict:
+    """{kernel name: (launches, total_ms, min_ms)} of the launches since the last collect."""
+    buf = C.create_string_buffer(1 << 16)
+    call("ody_profile_collect", buf, len(buf))
+    out = {}
+    for line in buf.value.decode().splitlines():
+        name, n, total, mn = line.split()
+        out[name] = (int(n), float(total), float(mn))
+    return out

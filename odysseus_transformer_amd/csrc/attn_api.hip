@@ -1,31 +1,6 @@
-// extern "C" entry points for attention and the error channel of the library.
-#include <cstdarg>
-#include <cstdio>
+// extern "C" entry points for attention.
 #include <cmath>
 #include "attn_params.h"
-
-namespace {
-thread_local char g_err[512] = "";
-}
-
-void ody_set_error(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
-  va_end(ap);
-}
-
-int ody_check_launch(const char* what) {
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) {
-    ody_set_error("%s: launch failed: %s", what, hipGetErrorString(e));
-    return ODY_ERR_LAUNCH;
-  }
-  return ODY_OK;
-}
-
-extern "C" const char* ody_last_error(void) { return g_err; }
-extern "C" int ody_version(void) { return 1; }
 
 namespace {
 

@@ -352,11 +352,11 @@ int launch(const AttnParams& p, hipStream_t st) {
     attr_set = true;
   }
   dim3 gk((p.Lk + 127) / 128, p.Hkv, p.B);
-  hipLaunchKernelGGL((attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, st, p);
+  ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
   int rc = ody_check_launch("attn_bwd_dkdv");
   if (rc) return rc;
   dim3 gq((p.Lq + 127) / 128, p.Hq, p.B);
-  hipLaunchKernelGGL((attn_bwd_dq_kernel<D>), gq, dim3(256), smem_q, st, p);
+  ODY_LAUNCH("attn_bwd_dq", st, (attn_bwd_dq_kernel<D>), gq, dim3(256), smem_q, p);
   return ody_check_launch("attn_bwd_dq");
 }
 

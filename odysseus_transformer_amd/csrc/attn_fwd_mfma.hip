@@ -243,7 +243,7 @@ int launch(const AttnParams& p, hipStream_t st) {
     attr_set = true;
   }
   dim3 grid((p.Lq + BM - 1) / BM, p.Hq, p.B);
-  hipLaunchKernelGGL((attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, st, p);
+  ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, p);
   return ody_check_launch("attn_fwd_mfma");
 }
 

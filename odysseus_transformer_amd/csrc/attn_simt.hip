@@ -274,21 +274,21 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnParams p) {
 template <typename T, int D>
 int launch_fwd(const AttnParams& p, hipStream_t st) {
   dim3 grid((p.Lq + SIMT_ROWS - 1) / SIMT_ROWS, p.Hq, p.B);
-  hipLaunchKernelGGL((attn_fwd_simt_kernel<T, D>), grid, dim3(SIMT_ROWS), 0, st, p);
+  ODY_LAUNCH("attn_fwd_simt", st, (attn_fwd_simt_kernel<T, D>), grid, dim3(SIMT_ROWS), 0, p);
   return ody_check_launch("attn_fwd_simt");
 }
 
 template <typename T, int D>
 int launch_bwd(const AttnParams& p, hipStream_t st) {
   dim3 gq((p.Lq + SIMT_ROWS - 1) / SIMT_ROWS, p.Hq, p.B);
-  hipLaunchKernelGGL((attn_bwd_dq_simt_kernel<T, D>), gq, dim3(SIMT_ROWS), 0, st, p);
+  ODY_LAUNCH("attn_bwd_dq_simt", st, (attn_bwd_dq_simt_kernel<T, D>), gq, dim3(SIMT_ROWS), 0, p);
   int rc = ody_check_launch("attn_bwd_dq_simt");
   if (rc) return rc;
   dim3 gk((p.Lk + SIMT_ROWS - 1) / SIMT_ROWS, p.Hkv, p.B);
-  hipLaunchKernelGGL((attn_bwd_dkv_simt_kernel<T, D, 0>), gk, dim3(SIMT_ROWS), 0, st, p);
+  ODY_LAUNCH("attn_bwd_dv_simt", st, (attn_bwd_dkv_simt_kernel<T, D, 0>), gk, dim3(SIMT_ROWS), 0, p);
   rc = ody_check_launch("attn_bwd_dv_simt");
   if (rc) return rc;
-  hipLaunchKernelGGL((attn_bwd_dkv_simt_kernel<T, D, 1>), gk, dim3(SIMT_ROWS), 0, st, p);
+  ODY_LAUNCH("attn_bwd_dk_simt", st, (attn_bwd_dkv_simt_kernel<T, D, 1>), gk, dim3(SIMT_ROWS), 0, p);
   return ody_check_launch("attn_bwd_dk_simt");
 }
 
@@ -296,7 +296,7 @@ template <typename T, int D>
 int launch_delta(const AttnParams& p, hipStream_t st) {
   constexpr int RPB = 256 / (D / Vec16B<T>::N);
   const int64_t total = (int64_t)p.B * p.Hq * p.Lq;
-  hipLaunchKernelGGL((attn_delta_kernel<T, D>), dim3((unsigned)((total + RPB - 1) / RPB)), dim3(256), 0, st, p);
+  ODY_LAUNCH("attn_delta", st, (attn_delta_kernel<T, D>), dim3((unsigned)((total + RPB - 1) / RPB)), dim3(256), 0, p);
   return ody_check_launch("attn_delta");
 }
 

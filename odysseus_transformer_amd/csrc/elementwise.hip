@@ -327,9 +327,9 @@ extern "C" int ody_rmsnorm_fwd(const void* x, const void* w, void* y, float* rst
   hipStream_t st = static_cast<hipStream_t>(stream);
   dim3 grid((T + 3) / 4);
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(rmsnorm_fwd_kernel<bf16>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
+               ODY_LAUNCH("rmsnorm_fwd", st, rmsnorm_fwd_kernel<bf16>, grid, dim3(256), 0, (const bf16*)x, (const bf16*)w,
                                   (bf16*)y, rstd, T, d, eps),
-               hipLaunchKernelGGL(rmsnorm_fwd_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)w,
+               ODY_LAUNCH("rmsnorm_fwd", st, rmsnorm_fwd_kernel<float>, grid, dim3(256), 0, (const float*)x, (const float*)w,
                                   (float*)y, rstd, T, d, eps));
   return ody_check_launch("rmsnorm_fwd");
 }
@@ -350,16 +350,16 @@ extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, 
   const int rpb = (T + nparts - 1) / nparts;
   const int nblocks = (T + rpb - 1) / rpb;  // <= nparts; rows of dw_partial beyond nblocks are not written
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(rmsnorm_bwd_kernel<bf16>, dim3(nblocks), dim3(256), 0, st, (const bf16*)x,
+               ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<bf16>, dim3(nblocks), dim3(256), 0, (const bf16*)x,
                                   (const bf16*)w, rstd, (const bf16*)dy, (bf16*)dx, dw_partial, T, d, rpb),
-               hipLaunchKernelGGL(rmsnorm_bwd_kernel<float>, dim3(nblocks), dim3(256), 0, st, (const float*)x,
+               ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<float>, dim3(nblocks), dim3(256), 0, (const float*)x,
                                   (const float*)w, rstd, (const float*)dy, (float*)dx, dw_partial, T, d, rpb));
   int rc = ody_check_launch("rmsnorm_bwd");
   if (rc || !dw) return rc;
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(colsum_kernel<bf16>, dim3((d + 255) / 256), dim3(256), 0, st, dw_partial, (bf16*)dw,
+               ODY_LAUNCH("colsum", st, colsum_kernel<bf16>, dim3((d + 255) / 256), dim3(256), 0, dw_partial, (bf16*)dw,
                                   nblocks, d),
-               hipLaunchKernelGGL(colsum_kernel<float>, dim3((d + 255) / 256), dim3(256), 0, st, dw_partial,
+               ODY_LAUNCH("colsum", st, colsum_kernel<float>, dim3((d + 255) / 256), dim3(256), 0, dw_partial,
                                   (float*)dw, nblocks, d));
   return ody_check_launch("rmsnorm_bwd_colsum");
 }
@@ -379,9 +379,9 @@ extern "C" int ody_rope(void* x, const int64_t* position_ids, const float* inv_f
   const int64_t total = (int64_t)B * L * (D / 2 / n);
   const float l2b = inv_freq ? 0.f : log2f(base);
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(rope_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st, (bf16*)x, position_ids,
+               ODY_LAUNCH("rope", st, rope_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, (bf16*)x, position_ids,
                                   inv_freq, B, L, n_rot, D, sx_b, sx_l, sx_h, l2b, inverse),
-               hipLaunchKernelGGL(rope_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st, (float*)x,
+               ODY_LAUNCH("rope", st, rope_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, (float*)x,
                                   position_ids, inv_freq, B, L, n_rot, D, sx_b, sx_l, sx_h, l2b, inverse));
   return ody_check_launch("rope");
 }
@@ -398,9 +398,9 @@ extern "C" int ody_swiglu_fwd(const void* gate_up, void* h, int T, int I, int64_
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = (int64_t)T * (I / n);
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(swiglu_fwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st,
+               ODY_LAUNCH("swiglu_fwd", st, swiglu_fwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0,
                                   (const bf16*)gate_up, (bf16*)h, T, I, ld_gu, ld_h),
-               hipLaunchKernelGGL(swiglu_fwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st,
+               ODY_LAUNCH("swiglu_fwd", st, swiglu_fwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0,
                                   (const float*)gate_up, (float*)h, T, I, ld_gu, ld_h));
   return ody_check_launch("swiglu_fwd");
 }
@@ -418,9 +418,9 @@ extern "C" int ody_swiglu_bwd(const void* gate_up, const void* dh, void* d_gate_
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = (int64_t)T * (I / n);
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(swiglu_bwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st,
+               ODY_LAUNCH("swiglu_bwd", st, swiglu_bwd_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0,
                                   (const bf16*)gate_up, (const bf16*)dh, (bf16*)d_gate_up, T, I, ld_gu, ld_dh, ld_dgu),
-               hipLaunchKernelGGL(swiglu_bwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st,
+               ODY_LAUNCH("swiglu_bwd", st, swiglu_bwd_kernel<float>, dim3(blocks_for(total)), dim3(256), 0,
                                   (const float*)gate_up, (const float*)dh, (float*)d_gate_up, T, I, ld_gu, ld_dh,
                                   ld_dgu));
   return ody_check_launch("swiglu_bwd");
@@ -437,9 +437,9 @@ extern "C" int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t total = (int64_t)B * L * H * (D / 4);
   ODY_BY_DTYPE(dtype,
-               hipLaunchKernelGGL(lse_merge_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, st, out_acc, lse_acc,
+               ODY_LAUNCH("lse_merge", st, lse_merge_kernel<bf16>, dim3(blocks_for(total)), dim3(256), 0, out_acc, lse_acc,
                                   (const bf16*)out_blk, lse_blk, B, L, H, D, sb_b, sb_l, sb_h),
-               hipLaunchKernelGGL(lse_merge_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, st, out_acc, lse_acc,
+               ODY_LAUNCH("lse_merge", st, lse_merge_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, out_acc, lse_acc,
                                   (const float*)out_blk, lse_blk, B, L, H, D, sb_b, sb_l, sb_h));
   return ody_check_launch("lse_merge");
 }

@@ -188,8 +188,9 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
     attr_set = true;
   }
   const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
-  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(256), smem, st, A, B, C, bias, M, N, K, lda, ldb, ldc,
-                     accumulate, tiles_m, tiles_n);
+  const char* name = A_KC ? (B_KC ? "gemm_bf16_nt" : "gemm_bf16_nn") : "gemm_bf16_tn";
+  ODY_LAUNCH(name, st, kern, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
+             accumulate, tiles_m, tiles_n);
   return ody_check_launch("gemm_bf16");
 }
 
@@ -274,7 +275,7 @@ extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const voi
     if (op == ODY_GEMM_NT) { sbk = 1; sbn = ldb; } else { sbk = ldb; sbn = 1; }
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     ODY_REQUIRE(grid.y <= 65535, ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d too large for the fp32 path", M);
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, st, (const float*)A, (const float*)B, (float*)C,
+    ODY_LAUNCH("gemm_f32", st, gemm_f32_kernel, grid, dim3(256), 0, (const float*)A, (const float*)B, (float*)C,
                        (const float*)bias, M, N, K, sam, sak, sbk, sbn, ldc, accumulate);
     return ody_check_launch("gemm_f32");
   }

@@ -24,6 +24,22 @@ void ody_set_error(const char* fmt, ...);
 // Returns ODY_OK or ODY_ERR_LAUNCH after a kernel launch (reads hipGetLastError).
 int ody_check_launch(const char* what);
 
+// Brackets one kernel launch with a pair of HIP events on the launch stream when the
+// timer is enabled (ody_profile_enable); costs one branch otherwise.
+struct OdyKernelScope {
+  OdyKernelScope(const char* name, hipStream_t st);
+  ~OdyKernelScope();
+  const char* name_;
+  hipStream_t st_;
+  hipEvent_t start_;
+};
+
+#define ODY_LAUNCH(name, st, kernel, grid, block, smem, ...)                      \
+  do {                                                                            \
+    OdyKernelScope ody_scope_(name, st);                                          \
+    hipLaunchKernelGGL(kernel, grid, block, smem, st, __VA_ARGS__);               \
+  } while (0)
+
 #define ODY_REQUIRE(cond, code, ...)        \
   do {                                      \
     if (!(cond)) {                          \

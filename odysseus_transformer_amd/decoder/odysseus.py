@@ -1,0 +1,266 @@
+"""Odysseus attention block and ZeRO-3 SwiGLU MLP (decoder/odysseus.py of the
+reference) on the gfx950 HIP library, plus the module patcher.
+
+Layout of one rank: the residual stream is the sequence shard (1, L/N, d); the
+attention block gathers the sequence, projects it onto this rank's heads
+(packed [q heads ; k heads ; v heads] rows of the column-split weight), applies
+RoPE with the FULL position ids, runs causal attention over the whole sequence,
+and row-splits the output projection; the MLP stays on the local tokens.
+
+The reference subclasses transformers' LlamaFlashAttention2, which current
+transformers no longer ship.  The class here is self-contained (reads the same
+config fields, owns its rotary table) and keeps the reference's constructor
+keywords, parameter names and shapes, and return convention.
+"""
+from __future__ import annotations
+
+import inspect
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from .. import ops
+from ..parallel_state import get_model_parallel_rank, get_model_parallel_world_size
+from ..utils.allgather import allgather_bsz1
+from ..utils.linear_tpsp import ColumnParallelLinear, ColumnParallelLinearAG, RowParallelLinearRS
+from ..utils.linear_zero3 import LinearZeRO3
+
+
+def _rope_theta(config) -> float:
+    params = getattr(config, "rope_parameters", None)
+    if isinstance(params, dict) and "rope_theta" in params:
+        return float(params["rope_theta"])
+    return float(getattr(config, "rope_theta", 10000.0))
+
+
+class PackedRoPEAttnFunc(torch.autograd.Function):
+    """RoPE + causal GQA attention on the packed projection, without a single copy.
+
+    qkv3 (1, L, (Hq + 2 Hkv) * D) is the output of the packed projection; its first
+    Hq + Hkv heads are rotated IN PLACE, attention reads q/k/v as head-axis slices
+    of that same buffer.  Backward writes dq/dk/dv straight into the slices of one
+    packed gradient buffer and un-rotates its q/k part in place.
+    """
+
+    @staticmethod
+    def forward(ctx, qkv3, n_heads, n_kv_heads, head_dim, position_ids, rope_base, softmax_scale):
+        B, L, _ = qkv3.shape
+        qkv = qkv3.view(B, L, n_heads + 2 * n_kv_heads, head_dim)
+        ops.rope_(qkv, n_heads + n_kv_heads, position_ids, rope_base)
+        ctx.mark_dirty(qkv3)
+        ctx.set_materialize_grads(False)  # no zero tensor for the rotated projection when nothing consumes it
+        a, b = n_heads, n_heads + n_kv_heads
+        out, lse = ops.attn_fwd(qkv[:, :, :a], qkv[:, :, a:b], qkv[:, :, b:], causal=True, scale=softmax_scale)
+        ctx.save_for_backward(qkv3, out, lse, position_ids)
+        ctx.dims = (n_heads, n_kv_heads, head_dim, rope_base, softmax_scale)
+        ctx.mark_non_differentiable(lse)
+        return qkv3, out, lse
+
+    @staticmethod
+    def backward(ctx, _dqkv_unused, dout, _dlse):
+        qkv3, out, lse, position_ids = ctx.saved_tensors
+        n_heads, n_kv_heads, head_dim, rope_base, softmax_scale = ctx.dims
+        B, L, _ = qkv3.shape
+        qkv = qkv3.view(B, L, n_heads + 2 * n_kv_heads, head_dim)
+        if dout is None:
+            dout = torch.zeros_like(out)
+        if dout.stride(3) != 1:
+            dout = dout.contiguous()
+        dqkv = torch.empty_like(qkv)
+        a, b = n_heads, n_heads + n_kv_heads
+        ops.attn_bwd(qkv[:, :, :a], qkv[:, :, a:b], qkv[:, :, b:], out, lse, dout, causal=True, scale=softmax_scale,
+                     dq=dqkv[:, :, :a], dk=dqkv[:, :, a:b], dv=dqkv[:, :, b:])
+        ops.rope_(dqkv, b, position_ids, rope_base, inverse=True)
+        if _dqkv_unused is not None:  # a consumer of the rotated projection itself (the KV cache does not differentiate)
+            dqkv = dqkv + _dqkv_unused.view_as(dqkv)
+        return dqkv.view_as(qkv3), None, None, None, None, None, None
+
+
+class LlamaFlashAttention2TPSP(nn.Module):
+    """Head-sharded causal attention over the gathered sequence
+    (decoder/odysseus.py:45-271).
+
+    Args (as the reference):
+        config, layer_idx: the Llama config and the index of the layer.
+        keep_master_weight_for_test: keep the unsplit weight of each sharded linear.
+        pack_weight: one packed QKV projection (default) or three separate ones.
+        sequence_parallel: the packed projection gathers the sequence itself and does
+            not save the gathered activation.
+    """
+
+    def __init__(self, config, layer_idx: Optional[int] = None, *, keep_master_weight_for_test=False,
+                 pack_weight=True, sequence_parallel=True):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.attention_dropout = getattr(config, "attention_dropout", 0.0)
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.head_dim = getattr(config, "head_dim", None) or self.hidden_size // self.num_heads
+        self.num_key_value_heads = getattr(config, "num_key_value_heads", None) or self.num_heads
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.max_position_embeddings = getattr(config, "max_position_embeddings", None)
+        self.rope_theta = _rope_theta(config)
+        self.is_causal = True
+
+        self.model_parallel_size = get_model_parallel_world_size()
+        self.local_rank = get_model_parallel_rank()
+        self.n_local_heads = self.num_heads // self.model_parallel_size
+        self.n_local_kv_heads = self.num_key_value_heads // self.model_parallel_size
+
+        self.q_proj = self.k_proj = self.v_proj = None
+        self.pack_weight = pack_weight
+        self.sequence_parallel = sequence_parallel
+        kw = dict(bias=False, gather_output=False, keep_master_weight_for_test=keep_master_weight_for_test)
+        if pack_weight:
+            cls = ColumnParallelLinearAG if sequence_parallel else ColumnParallelLinear
+            self.qkv_proj = cls(self.hidden_size, (self.num_heads + 2 * self.num_key_value_heads) * self.head_dim, **kw)
+        else:
+            self.q_proj = ColumnParallelLinear(self.hidden_size, self.num_heads * self.head_dim, **kw)
+            self.k_proj = ColumnParallelLinear(self.hidden_size, self.num_key_value_heads * self.head_dim, **kw)
+            self.v_proj = ColumnParallelLinear(self.hidden_size, self.num_key_value_heads * self.head_dim, **kw)
+        self.o_proj = RowParallelLinearRS(self.num_heads * self.head_dim, self.hidden_size, bias=False,
+                                          input_is_parallel=True,
+                                          keep_master_weight_for_test=keep_master_weight_for_test)
+        # arity of the tuple forward() returns: 3 as the reference (attn_output, attn_weights,
+        # past_key_value); the patcher lowers it to 2 for host decoder layers that unpack two values
+        self.return_arity = 3
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                position_ids: Optional[torch.LongTensor] = None, past_key_value=None, output_attentions: bool = False,
+                use_cache: bool = False, cache_position: Optional[torch.LongTensor] = None, **kwargs):
+        if past_key_value is None:
+            past_key_value = kwargs.get("past_key_values")
+        if type(past_key_value).__name__ == "StaticCache":
+            raise ValueError(
+                "`static` cache implementation is not compatible with `attn_implementation==flash_attention_2` "
+                "make sure to use `sdpa` in the mean time, and open an issue at "
+                "https://github.com/huggingface/transformers")
+        if attention_mask is not None:
+            raise NotImplementedError("padding masks are not supported: the training loop passes attention_mask=None")
+        bsz, local_q_len, _ = hidden_states.size()
+        assert bsz == 1, f"bsz: {bsz}"
+        if self.training and self.attention_dropout != 0.0:
+            raise NotImplementedError("attention dropout is not implemented (the reference trains with 0.0)")
+        scale = 1.0 / math.sqrt(self.head_dim)
+        nh, nkv, D = self.n_local_heads, self.n_local_kv_heads, self.head_dim
+
+        if self.pack_weight:
+            q_len = local_q_len * get_model_parallel_world_size()
+            if not self.sequence_parallel:
+                hidden_states = allgather_bsz1(hidden_states)
+            qkv3, attn_output, _ = PackedRoPEAttnFunc.apply(self.qkv_proj(hidden_states), nh, nkv, D, position_ids,
+                                                            self.rope_theta, scale)
+            if past_key_value is not None:
+                qkv = qkv3.detach().view(bsz, q_len, nh + 2 * nkv, D)
+                self._update_cache(past_key_value, qkv[:, :, nh:nh + nkv], qkv[:, :, nh + nkv:], q_len, cache_position)
+        else:
+            hidden_states = allgather_bsz1(hidden_states)
+            bsz, q_len, _ = hidden_states.size()
+            q = self.q_proj(hidden_states).view(bsz, q_len, nh, D)
+            k = self.k_proj(hidden_states).view(bsz, q_len, nkv, D)
+            v = self.v_proj(hidden_states).view(bsz, q_len, nkv, D)
+            q = ops.apply_rope_packed(q, nh, position_ids, self.rope_theta)
+            k = ops.apply_rope_packed(k, nkv, position_ids, self.rope_theta)
+            if past_key_value is not None:
+                self._update_cache(past_key_value, k.detach(), v.detach(), q_len, cache_position)
+            attn_output = ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+
+        attn_output = attn_output.reshape(bsz, q_len, nh * D)
+        attn_output = self.o_proj(attn_output)
+        if self.return_arity == 2:
+            return attn_output, None
+        return attn_output, None, past_key_value
+
+    def _update_cache(self, cache, k, v, q_len, cache_position):
+        """Hands the rotated keys and the values of a prefill to the caller's cache, as
+        decoder/odysseus.py:215-220 does.  Attending to EARLIER cache content is the
+        decoding path, which this training-side module does not implement."""
+        k_all, _ = cache.update(k.transpose(1, 2), v.transpose(1, 2), self.layer_idx,
+                                {"cache_position": cache_position})
+        if k_all.shape[-2] != q_len:
+            raise NotImplementedError("attention over a non-empty KV cache (incremental decoding) is not implemented")
+
+
+class LlamaMLPZeRO(nn.Module):
+    """SwiGLU MLP on the local tokens with ZeRO-3 sharded weights
+    (decoder/odysseus.py:274-295): gate = rows [0, i) and up = rows [i, 2i) of the
+    full gate_up weight."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.hidden_size = config.hidden_size
+        self.intermediate_size = config.intermediate_size
+        self.gate_up_proj = LinearZeRO3(self.hidden_size, self.intermediate_size * 2, bias=False)
+        self.down_proj = LinearZeRO3(self.intermediate_size, self.hidden_size, bias=False)
+        act = getattr(config, "hidden_act", "silu")
+        if act != "silu":
+            raise NotImplementedError(f"hidden_act={act!r}: only the SiLU gate of Llama is implemented")
+        self.act_fn = torch.nn.functional.silu  # kept as an attribute for introspection; the fused kernel applies it
+
+    def forward(self, x):
+        if getattr(self.config, "pretraining_tp", 1) > 1:
+            raise NotImplementedError("pretraining_tp > 1 is not supported yet.")
+        return self.down_proj(ops.swiglu(self.gate_up_proj(x)))
+
+
+class LlamaRMSNorm(nn.Module):
+    """RMSNorm with fp32 statistics (the input_layernorm / post_attention_layernorm the
+    decoder layer calls, decoder/ring.py:67,84)."""
+
+    def __init__(self, hidden_size, eps=1e-6):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def forward(self, hidden_states):
+        return ops.rmsnorm(hidden_states, self.weight, self.variance_epsilon)
+
+
+class OdysseusDecoderLayer(nn.Module):
+    """h = x + attn(rms(x)); y = h + mlp(rms(h)) (the wiring at decoder/ring.py:65-86)."""
+
+    def __init__(self, config, layer_idx: int = 0):
+        super().__init__()
+        self.hidden_size = config.hidden_size
+        eps = getattr(config, "rms_norm_eps", 1e-6)
+        self.self_attn = LlamaFlashAttention2TPSP(config, layer_idx)
+        self.mlp = LlamaMLPZeRO(config)
+        self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps)
+        self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
+
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, **kwargs):
+        residual = hidden_states
+        hidden_states = self.self_attn(self.input_layernorm(hidden_states), attention_mask=attention_mask,
+                                       position_ids=position_ids)[0]
+        hidden_states = residual + hidden_states
+        residual = hidden_states
+        hidden_states = self.mlp(self.post_attention_layernorm(hidden_states))
+        return residual + hidden_states
+
+
+def _host_layer_unpacks_two(layer) -> bool:
+    """Recent transformers decoder layers pass `position_embeddings` and unpack
+    `hidden_states, _ = self.self_attn(...)`; older ones unpack three values."""
+    try:
+        return "position_embeddings" in inspect.signature(layer.forward).parameters
+    except (TypeError, ValueError):
+        return False
+
+
+def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True):
+    """Swaps every layer's attention (and, by default, MLP) for the Odysseus modules
+    (decoder/odysseus.py:298-309).  As in the reference the new modules are freshly
+    initialised: pretrained attention / MLP weights are not carried over."""
+    for i in range(model.config.num_hidden_layers):
+        layer = model.model.layers[i]
+        new_module = LlamaFlashAttention2TPSP(model.config, i).to(model.dtype)
+        if _host_layer_unpacks_two(layer):
+            new_module.return_arity = 2
+        layer.self_attn = new_module
+        if use_zero3_linear:
+            layer.mlp = LlamaMLPZeRO(model.config).to(model.dtype)
+    print("Applied Odysseus patch for LlamaFlashAttn")

@@ -1,0 +1,143 @@
+"""GPU parity of the module layer: attention block, MLP and the whole decoder layer
+(forward and every gradient) against the CPU oracle with the same seeded inputs."""
+import types
+import zlib
+
+import pytest
+import torch
+
+from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
+import odysseus_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _config(d, H, Hkv, D, i):
+    return types.SimpleNamespace(hidden_size=d, num_attention_heads=H, num_key_value_heads=Hkv, head_dim=D,
+                                 intermediate_size=i, hidden_act="silu", attention_dropout=0.0, rms_norm_eps=1e-6,
+                                 rope_theta=10000.0, max_position_embeddings=1 << 20, pretraining_tp=1,
+                                 num_hidden_layers=1)
+
+
+def _params(d, H, Hkv, D, i, dtype, seed=0):
+    p = {
+        "ln1": 1.0 + randn((d,), seed + 1, std=0.02),
+        "w_qkv": randn(((H + 2 * Hkv) * D, d), seed + 2, std=0.02),
+        "w_o": randn((d, H * D), seed + 3, std=0.02),
+        "ln2": 1.0 + randn((d,), seed + 4, std=0.02),
+        "w_gate_up": randn((2 * i, d), seed + 5, std=0.02),
+        "w_down": randn((d, i), seed + 6, std=0.02),
+    }
+    return {k: v.to(dtype) for k, v in p.items()}
+
+
+def _load(layer, p, dev):
+    layer = layer.to(dev)
+    with torch.no_grad():
+        layer.input_layernorm.weight.copy_(p["ln1"])
+        layer.self_attn.qkv_proj.weight.copy_(p["w_qkv"])
+        layer.self_attn.o_proj.weight.copy_(p["w_o"])
+        layer.post_attention_layernorm.weight.copy_(p["ln2"])
+        layer.mlp.gate_up_proj.weight.copy_(p["w_gate_up"])
+        layer.mlp.down_proj.weight.copy_(p["w_down"])
+    return layer
+
+
+LAYER_CASES = [
+    # name, L, d, H, Hkv, D, i, dtype
+    ("cfg1_fp32", 2048, 512, 8, 8, 64, 1376, torch.float32),       # the reference's CPU-runnable configuration
+    ("bf16_mha", 1024, 512, 4, 4, 128, 1408, torch.bfloat16),
+    ("bf16_gqa_ragged", 520, 1024, 4, 1, 128, 2816, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", LAYER_CASES, ids=lambda c: c[0])
+def test_decoder_layer_fwd_bwd(case, dev):
+    from odysseus_transformer_amd.decoder.odysseus import OdysseusDecoderLayer
+    name, L, d, H, Hkv, D, i, dtype = case
+    print(f"layer case {name}", flush=True)
+    tol = TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
+    p = _params(d, H, Hkv, D, i, dtype)
+    x = randn((1, L, d), 100, dtype=dtype)
+    dy = randn((1, L, d), 101, dtype=dtype)
+    pf = {k: v.float() for k, v in p.items()}
+    y_ref, g_ref = oracle.decoder_layer_fwd_bwd(x.float(), pf, dy.float(), H, Hkv, D)
+
+    layer = _load(OdysseusDecoderLayer(_config(d, H, Hkv, D, i)).to(dtype), p, dev)
+    xg = x.to(dev).requires_grad_(True)
+    pos = torch.arange(L, device=dev)[None]
+    y = layer(xg, position_ids=pos)
+    y.backward(dy.to(dev))
+    torch.cuda.synchronize()
+    assert rel_err(y, y_ref) <= tol, "y"
+    got = {
+        "x": xg.grad, "ln1": layer.input_layernorm.weight.grad, "w_qkv": layer.self_attn.qkv_proj.weight.grad,
+        "w_o": layer.self_attn.o_proj.weight.grad, "ln2": layer.post_attention_layernorm.weight.grad,
+        "w_gate_up": layer.mlp.gate_up_proj.weight.grad, "w_down": layer.mlp.down_proj.weight.grad,
+    }
+    for k, v in got.items():
+        assert rel_err(v, g_ref[k]) <= tol, f"grad {k}: {rel_err(v, g_ref[k])}"
+
+
+def test_attention_block_unpacked_equals_packed(dev):
+    """Three separate projections with rows [q ; k ; v] of the packed weight give the
+    packed module's output (the identity the reference's tests rely on for w1w3)."""
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    d, H, Hkv, D, L = 512, 4, 2, 128, 384
+    cfg = _config(d, H, Hkv, D, 1024)
+    dt = torch.bfloat16
+    packed = LlamaFlashAttention2TPSP(cfg, 0).to(dt).to(dev)
+    unpacked = LlamaFlashAttention2TPSP(cfg, 0, pack_weight=False).to(dt).to(dev)
+    w = randn(((H + 2 * Hkv) * D, d), 7, std=0.02, dtype=dt).to(dev)
+    wo = randn((d, H * D), 8, std=0.02, dtype=dt).to(dev)
+    with torch.no_grad():
+        packed.qkv_proj.weight.copy_(w)
+        packed.o_proj.weight.copy_(wo)
+        unpacked.q_proj.weight.copy_(w[:H * D])
+        unpacked.k_proj.weight.copy_(w[H * D:(H + Hkv) * D])
+        unpacked.v_proj.weight.copy_(w[(H + Hkv) * D:])
+        unpacked.o_proj.weight.copy_(wo)
+    x = randn((1, L, d), 9, dtype=dt).to(dev)
+    ya, none_a, cache_a = packed(x)
+    yb = unpacked(x)[0]
+    assert none_a is None and cache_a is None
+    assert rel_err(ya, yb.float()) <= 1e-2
+    y_ref, _ = oracle.attention_block(x.float().cpu(), w.float().cpu(), wo.float().cpu(), H, Hkv, D)
+    assert rel_err(ya, y_ref) <= TOL_BF16
+
+
+def test_patched_hf_llama_runs_and_matches_oracle(dev):
+    """apply_odysseus_attn_patch_llama on a small transformers Llama: logits and the
+    gradient of the token embedding equal the oracle's composition of the same layers."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from odysseus_transformer_amd.decoder.odysseus import apply_odysseus_attn_patch_llama
+    torch.manual_seed(0)
+    cfg = LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                      num_key_value_heads=1, head_dim=128, vocab_size=128, max_position_embeddings=2048,
+                      rms_norm_eps=1e-6)
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16)
+    apply_odysseus_attn_patch_llama(model)
+    with torch.no_grad():
+        for n, prm in model.named_parameters():
+            if "mlp" in n or "self_attn" in n:
+                prm.copy_(randn(tuple(prm.shape), zlib.crc32(n.encode()) % 1000, std=0.02))
+    model = model.to(dev)
+    L = 200
+    ids = torch.randint(0, 128, (1, L), generator=torch.Generator().manual_seed(1))
+    pos = torch.arange(L)[None]
+    logits = model(ids.to(dev), position_ids=pos.to(dev), use_cache=False).logits
+    # oracle composition
+    sd = {k: v.float().cpu() for k, v in model.state_dict().items()}
+    h = sd["model.embed_tokens.weight"][ids]
+    for l in range(2):
+        pre = f"model.layers.{l}."
+        p = {"ln1": sd[pre + "input_layernorm.weight"], "w_qkv": sd[pre + "self_attn.qkv_proj.weight"],
+             "w_o": sd[pre + "self_attn.o_proj.weight"], "ln2": sd[pre + "post_attention_layernorm.weight"],
+             "w_gate_up": sd[pre + "mlp.gate_up_proj.weight"], "w_down": sd[pre + "mlp.down_proj.weight"]}
+        h = oracle.decoder_layer_fwd(h, p, 2, 1, 128)
+    ref = oracle.linear_fwd(oracle.rmsnorm(h, sd["model.norm.weight"]), sd["lm_head.weight"])
+    assert rel_err(logits, ref) <= TOL_BF16
+    logits.float().square().mean().backward()
+    assert model.model.layers[0].self_attn.qkv_proj.weight.grad is not None
+    assert torch.isfinite(model.model.embed_tokens.weight.grad).all()
