@@ -66,14 +66,18 @@ int ody_profile_collect(char* out, size_t cap);
  *                      sees no key (its out row is 0).
  * GQA: q head h reads kv head h / (Hq / Hkv).  causal != 0 masks key j for
  * query i when j > i + (Lk - Lq).  D in {64, 128}.
+ * workspace: ody_attn_fwd_workspace_bytes(...) bytes, 256-byte aligned (the bf16
+ * head_dim-128 kernel keeps a transposed copy of V there; 0 bytes = may be NULL).
  */
+size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                  int B, int Lq, int Lk, int Hq, int Hkv, int D,
                  int64_t sq_b, int64_t sq_l, int64_t sq_h,
                  int64_t sk_b, int64_t sk_l, int64_t sk_h,
                  int64_t sv_b, int64_t sv_l, int64_t sv_h,
                  int64_t so_b, int64_t so_l, int64_t so_h,
-                 float scale, int causal, int dtype, void* stream);
+                 float scale, int causal, int dtype,
+                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* Backward of the above (flash_attn's backward as run by autograd through
  * decoder/odysseus.py:256-263).  `out` and `lse` are the forward results -- or,
@@ -83,9 +87,10 @@ int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* 
  * head are summed over its query-head group inside the kernel (deterministic,
  * no atomics).  If accumulate_dq != 0 the kernel adds into dq (fp32 dq_accum
  * layout not needed: the add happens in fp32 before rounding once).
- * workspace: ody_attn_bwd_workspace_bytes(B, Lq, Hq) bytes, 256-byte aligned.
+ * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
+ * the bf16 head_dim-128 kernels the transposed copies of K, Q and dO).
  */
-size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Hq);
+size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
                  const void* dout, void* dq, void* dk, void* dv,
                  int B, int Lq, int Lk, int Hq, int Hkv, int D,

@@ -10,7 +10,8 @@ int check_common(const char* who, int B, int Lq, int Lk, int Hq, int Hkv, int D,
   ODY_REQUIRE(Hq % Hkv == 0, ODY_ERR_BAD_SHAPE, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
   ODY_REQUIRE(D == 64 || D == 128, ODY_ERR_UNSUPPORTED, "%s: head_dim %d not built (64, 128)", who, D);
   ODY_REQUIRE(dtype == ODY_BF16 || dtype == ODY_F32, ODY_ERR_UNSUPPORTED, "%s: dtype %d unknown", who, dtype);
-  ODY_REQUIRE(B <= 65535 && Hq <= 65535, ODY_ERR_BAD_SHAPE, "%s: B and Hq must fit a grid dimension", who);
+  ODY_REQUIRE((int64_t)B * Hq * ((Lq + 63) / 64 + (Lk + 63) / 64) < (int64_t)1 << 31, ODY_ERR_BAD_SHAPE,
+              "%s: too many blocks for one launch", who);
   return ODY_OK;
 }
 
@@ -28,13 +29,16 @@ int check_tensor(const char* who, const char* name, const void* ptr, const AttnS
 
 }  // namespace
 
+extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
+
 extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                             int B, int Lq, int Lk, int Hq, int Hkv, int D,
                             int64_t sq_b, int64_t sq_l, int64_t sq_h,
                             int64_t sk_b, int64_t sk_l, int64_t sk_h,
                             int64_t sv_b, int64_t sv_l, int64_t sv_h,
                             int64_t so_b, int64_t so_l, int64_t so_h,
-                            float scale, int causal, int dtype, void* stream) {
+                            float scale, int causal, int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream) {
   int rc = check_common("ody_attn_fwd", B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
   AttnParams p{};
@@ -51,14 +55,34 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
   ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_fwd: lse is NULL");
   ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_fwd: scale must be positive");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && D == 128) {
+    const size_t need = ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype);
+    ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_fwd: workspace is NULL");
+    ODY_REQUIRE(workspace_bytes >= need, ODY_ERR_WORKSPACE, "ody_attn_fwd: workspace of %zu bytes, %zu needed",
+                workspace_bytes, need);
+    ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
+                "ody_attn_fwd: workspace must be 256-byte aligned");
+    return ody_launch_attn_fwd_pipe(p, workspace, st);
+  }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
   return ody_launch_attn_fwd_simt(p, D, dtype, st);
 }
 
-extern "C" size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Hq) {
-  if (B <= 0 || Lq <= 0 || Hq <= 0) return 0;
-  const size_t n = (size_t)B * Lq * Hq * sizeof(float);
-  return (n + 255) & ~(size_t)255;
+extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
+  if (B <= 0 || Lq <= 0 || Lk <= 0 || Hq <= 0 || Hkv <= 0) return 0;
+  if (dtype == ODY_BF16 && D == 128) return (ody_attn_fwd_pipe_workspace(B, Lq, Lk, Hq, Hkv) + 255) & ~(size_t)255;
+  return 0;
+}
+
+namespace {
+size_t delta_bytes(int B, int Lq, int Hq) { return ((size_t)B * Lq * Hq * sizeof(float) + 255) & ~(size_t)255; }
+}
+
+extern "C" size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
+  if (B <= 0 || Lq <= 0 || Lk <= 0 || Hq <= 0 || Hkv <= 0) return 0;
+  size_t n = delta_bytes(B, Lq, Hq);
+  if (dtype == ODY_BF16 && D == 128) n += ody_attn_bwd_pipe_workspace(B, Lq, Lk, Hq, Hkv);
+  return n;
 }
 
 extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
@@ -98,14 +122,16 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
   ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_bwd: lse is NULL");
   ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_bwd: scale must be positive");
   ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_bwd: workspace is NULL");
-  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Hq), ODY_ERR_WORKSPACE,
+  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype), ODY_ERR_WORKSPACE,
               "ody_attn_bwd: workspace of %zu bytes, %zu needed", workspace_bytes,
-              ody_attn_bwd_workspace_bytes(B, Lq, Hq));
+              ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype));
   ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
               "ody_attn_bwd: workspace must be 256-byte aligned");
   p.delta = static_cast<float*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if ((rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
+  if (dtype == ODY_BF16 && D == 128)
+    return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
   if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
   return ody_launch_attn_bwd_simt(p, D, dtype, st);
 }

@@ -82,8 +82,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnParams p) 
   float* Ds = Ls + 2 * BQ;                            // [2][BQ]  delta, same order
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
-  const int hk = blockIdx.y, b = blockIdx.z;
-  const int n0 = blockIdx.x * BN, wn0 = n0 + wave * WK, key = wn0 + i;
+  const BlockCoord bc = ody_block_coord(p.Hkv, p.B);   // rank 0 = first key block = most query tiles
+  const int hk = bc.h, b = bc.b;
+  const int n0 = bc.rank * BN, wn0 = n0 + wave * WK, key = wn0 + i;
   const bf16* kp = static_cast<const bf16*>(p.k) + b * p.sk.b + hk * p.sk.h;
   const bf16* vp = static_cast<const bf16*>(p.v) + b * p.sv.b + hk * p.sv.h;
 
@@ -226,9 +227,10 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
   bf16* Vs = Ks + 2 * BN * P;                    // [2][BN][P]
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
-  const int nqb = gridDim.x;
-  const int qblk = p.causal ? (nqb - 1 - (int)blockIdx.x) : (int)blockIdx.x;
-  const int h = blockIdx.y, b = blockIdx.z, hk = h / p.group;
+  const BlockCoord bc = ody_block_coord(p.Hq, p.B);
+  const int nqb = gridDim.x / (p.Hq * p.B);
+  const int qblk = p.causal ? (nqb - 1 - bc.rank) : bc.rank;   // heaviest blocks first
+  const int h = bc.h, b = bc.b, hk = h / p.group;
   const int q0 = qblk * BM, wq0 = q0 + wave * WQ, qi = wq0 + i;
   const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
   const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
@@ -351,11 +353,11 @@ int launch(const AttnParams& p, hipStream_t st) {
     }
     attr_set = true;
   }
-  dim3 gk((p.Lk + 127) / 128, p.Hkv, p.B);
+  dim3 gk(((p.Lk + 127) / 128) * p.Hkv * p.B);
   ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
   int rc = ody_check_launch("attn_bwd_dkdv");
   if (rc) return rc;
-  dim3 gq((p.Lq + 127) / 128, p.Hq, p.B);
+  dim3 gq(((p.Lq + 127) / 128) * p.Hq * p.B);
   ODY_LAUNCH("attn_bwd_dq", st, (attn_bwd_dq_kernel<D>), gq, dim3(256), smem_q, p);
   return ody_check_launch("attn_bwd_dq");
 }

@@ -25,7 +25,8 @@
 namespace {
 
 template <int D, int QT>
-__global__ __launch_bounds__(256) void attn_fwd_mfma_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams p, const int* __restrict__ flags,
+                                                               int flag_block) {
   constexpr int BN = 64, WQ = 32 * QT, BM = 4 * WQ;
   constexpr int KP = D + 8;    // K tile row pitch (elements): 16-byte reads of 16 rows hit 64 distinct banks
   constexpr int VP = D + 32;   // V tile row pitch: 4 rows x 32 columns of a transpose read hit distinct banks
@@ -38,10 +39,16 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_kernel(const AttnParams p) 
   bf16* Vs = Ks + 2 * BN * KP;                             // [2][BN][VP]
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
-  const int nqb = gridDim.x;
-  const int qblk = p.causal ? (nqb - 1 - (int)blockIdx.x) : (int)blockIdx.x;  // heaviest blocks first
-  const int h = blockIdx.y, b = blockIdx.z, hk = h / p.group;
+  const BlockCoord bc = ody_block_coord(p.Hq, p.B);
+  const int nqb = gridDim.x / (p.Hq * p.B);
+  const int qblk = p.causal ? (nqb - 1 - bc.rank) : bc.rank;   // heaviest blocks first
+  const int h = bc.h, b = bc.b, hk = h / p.group;
   const int q0 = qblk * BM, wq0 = q0 + wave * WQ;
+  // restricted run: only query blocks whose flag is set (the flags cover blocks of flag_block rows)
+  if (flags != nullptr) {
+    const int nfb = (p.Lq + flag_block - 1) / flag_block;
+    if (flags[((int64_t)b * p.Hq + h) * nfb + q0 / flag_block] == 0) return;
+  }
 
   const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
   const bf16* kp = static_cast<const bf16*>(p.k) + b * p.sk.b + hk * p.sk.h;
@@ -229,7 +236,7 @@ __global__ __launch_bounds__(256) void attn_fwd_mfma_kernel(const AttnParams p) 
 }
 
 template <int D, int QT>
-int launch(const AttnParams& p, hipStream_t st) {
+int launch(const AttnParams& p, const int* flags, int flag_block, hipStream_t st) {
   constexpr int BN = 64, BM = 4 * 32 * QT;
   constexpr size_t smem = (size_t)2 * BN * ((D + 8) + (D + 32)) * sizeof(bf16);
   static bool attr_set = false;
@@ -242,16 +249,20 @@ int launch(const AttnParams& p, hipStream_t st) {
     }
     attr_set = true;
   }
-  dim3 grid((p.Lq + BM - 1) / BM, p.Hq, p.B);
-  ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, p);
+  dim3 grid(((p.Lq + BM - 1) / BM) * p.Hq * p.B);
+  ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, p, flags, flag_block);
   return ody_check_launch("attn_fwd_mfma");
 }
 
 }  // namespace
 
 int ody_launch_attn_fwd_mfma(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 128) return launch<128, 1>(p, st);
-  if (D == 64) return launch<64, 1>(p, st);
+  if (D == 128) return launch<128, 1>(p, nullptr, 1, st);
+  if (D == 64) return launch<64, 1>(p, nullptr, 1, st);
   ody_set_error("attn_fwd: head_dim %d not built (64, 128)", D);
   return ODY_ERR_UNSUPPORTED;
+}
+
+int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st) {
+  return launch<128, 1>(p, flags, block, st);
 }

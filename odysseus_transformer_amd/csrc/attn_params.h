@@ -26,8 +26,36 @@ struct AttnParams {
   AttnStrides sq, sk, sv, so, sdo, sdq, sdk, sdv;
 };
 
+// Block order of the attention kernels: a 1-D grid whose linear id runs over (head, batch)
+// fastest and over the row-block rank slowest.  With causal masking the work of a row block
+// grows with its index, so rank 0 is the heaviest block: the dispatcher then hands out the
+// heavy blocks of ALL heads first and the light ones fill the tail (a (blocks, heads) grid
+// would start with every block of head 0, light ones included).  Consecutive ids also map
+// to consecutive XCDs, so with 4 or 8 heads each XCD works on one head and its workgroups
+// walk the same K / V (or Q / dO) tiles at the same time, sharing them through its L2.
+struct BlockCoord { int rank, h, b; };
+#ifdef __HIPCC__
+__device__ __forceinline__ BlockCoord ody_block_coord(int H, int B) {
+  const int id = blockIdx.x, hb = id % (H * B);
+  return BlockCoord{id / (H * B), hb % H, hb / H};
+}
+#endif
+
 // Launchers (one per translation unit); each returns an ody_status.
 int ody_launch_attn_fwd_mfma(const AttnParams& p, int D, hipStream_t st);
+// head_dim 128 only; workspace of ody_attn_fwd_pipe_workspace(...) bytes
+int ody_launch_attn_fwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
+// transposed 64-row tile images of a (B, L, H, 128) bf16 matrix (attn_tile.h)
+size_t ody_attn_images_bytes(int B, int L, int H);
+// also zeroes `nflags` ints at `flags` (may be NULL)
+int ody_launch_attn_images(const void* src, const AttnStrides& s, int B, int L, int H, void* dst, int* flags,
+                           int nflags, hipStream_t st);
+size_t ody_attn_fwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
+// the online-rescaling forward kernel restricted to query blocks of `block` rows whose flag is set
+int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st);
+// head_dim 128 only; workspace of ody_attn_bwd_pipe_workspace(...) bytes (p.delta is set separately)
+size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
+int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st);
 int ody_launch_attn_fwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);
 int ody_launch_attn_bwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);

@@ -1,0 +1,147 @@
+// LDS tiles of the head_dim-128 attention kernels: 64 rows x 128 bf16, filled by
+// direct global->LDS loads and read both row-wise (16-byte reads) and transposed
+// (ds_read_b64_tr_b16) without bank conflicts, with purely additive addressing.
+//
+// A direct load (global_load_lds_dwordx4) makes the 64 lanes of a wavefront write
+// 64 consecutive 16-byte slots of LDS, each lane fetching from its own global
+// address.  One such load brings a GROUP of 4 consecutive tile rows (4 x 256 B);
+// inside the group the slots are chunk-major: slot = chunk * 4 + (row & 3), where a
+// chunk is 8 consecutive bf16 of a row.  Groups are 1040 bytes apart (1024 + 16 of
+// padding).  Hence, in elements,
+//
+//     offset(row, col) = (row >> 2) * 520 + (col >> 3) * 32 + (row & 3) * 8 + (col & 7)
+//
+//  * row-wise operand: the 16 lanes that are served together read the same chunk
+//    of rows 4*i + b (i = 0..15, b fixed): their addresses are 1040 bytes apart,
+//    i.e. 4 banks apart -> 64 distinct banks;
+//  * transposed operand: one 16-lane block reads 4 rows of 4 consecutive groups
+//    (same b) x 2 chunks x 2 halves: banks 4t + 16x + 2y (+0/1), all distinct.
+//
+// To make both patterns line up, row rho (0..31) of a 32-row MFMA operand of
+// sub-tile kt (0/1) is tile row  4*(rho & 15) + (rho >> 4) + 2*kt.
+#pragma once
+#include "ody_common.h"
+
+namespace tile128 {
+
+constexpr int ROWS = 64;
+constexpr int GROUP_ELEMS = 520;                 // 1040 bytes
+constexpr int TILE_ELEMS = 16 * GROUP_ELEMS;     // 8320 elements = 16640 bytes
+constexpr int TILE_BYTES = TILE_ELEMS * 2;
+
+// tile row of MFMA row rho of sub-tile kt
+__device__ __forceinline__ int tile_row(int rho, int kt) { return 4 * (rho & 15) + (rho >> 4) + 2 * kt; }
+
+// tile row held in accumulator register r of lane group g (accumulator rows are
+// rho = 8*(r>>2) + 4g + (r&3))
+__device__ __forceinline__ int acc_tile_row(int r, int g, int kt) {
+  return 32 * ((r >> 2) & 1) + 16 * g + 4 * (r & 3) + (r >> 3) + 2 * kt;
+}
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef __attribute__((address_space(1))) const void* global_void_ptr;
+
+// Issues this thread's share of the direct loads of one 64 x 128 tile: 4 loads of
+// 16 bytes (256 threads).  `base` points at row 0 of the matrix for this (batch, head);
+// rows at or beyond `nrows` re-read row nrows-1 (finite filler that the caller masks).
+__device__ __forceinline__ void load_tile_async(bf16* lds_tile, const bf16* base, int64_t row_stride, int row0,
+                                                int nrows, int wave, int lane) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int grp = 4 * j + wave;
+    int row = row0 + 4 * grp + (lane & 3);
+    row = row < nrows ? row : nrows - 1;
+    const bf16* src = base + (int64_t)row * row_stride + 8 * (lane >> 2);
+    __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + grp * GROUP_ELEMS), 16, 0, 0);
+  }
+}
+
+// Per-lane element offset of the row-wise operand: MFMA row i, k = 8g..8g+7 of k-step 0,
+// sub-tile 0.  Add ks*64 + kt*16 elements for k-step ks of sub-tile kt.
+__device__ __forceinline__ int row_frag_base(int g, int i) { return (i & 15) * GROUP_ELEMS + g * 32 + (i >> 4) * 8; }
+
+__device__ __forceinline__ bf16x8 row_frag(const bf16* tile, int base, int ks, int kt) {
+  return *reinterpret_cast<const bf16x8*>(tile + base + ks * 64 + kt * 16);
+}
+
+// Per-lane element offset of the transposed operand: this lane supplies the address of
+// 4 consecutive columns of one row; after the transpose read the lane holds column
+// 32*dt + i of the rows that k-step ss of sub-tile kt contracts over (first half: rows
+// of groups 4g..4g+3, second half: +8 groups).  Add dt*128 + (ss + 2*kt)*8 (+ 8 groups).
+__device__ __forceinline__ int tr_frag_base(int g, int i) {
+  return (4 * g + ((i & 15) >> 2)) * GROUP_ELEMS + (2 * (i >> 4) + ((i & 3) >> 1)) * 32 + 4 * (i & 1);
+}
+
+__device__ __forceinline__ bf16x8 tr_frag(const bf16* tile, int base, int dt, int ss, int kt) {
+  const bf16* p = tile + base + dt * 128 + (ss + 2 * kt) * 8;
+  return concat4(lds_read_tr16(p), lds_read_tr16(p + 8 * GROUP_ELEMS));
+}
+
+// ---------------------------------------------------------------------------------
+// Transposed tiles ("images").  An operand that an MFMA contracts over its ROW index
+// (V in O^T += V^T P^T, Q and dO in the dK/dV products, K in dQ^T += K^T dS^T) is not
+// read with the transpose instruction -- ds_read_b64_tr_b16 delivers half the LDS
+// bandwidth of a 16-byte read -- but from a transposed copy that a small pre-pass
+// writes to the workspace, one 16 KB image per 64-row tile, already in the order the
+// LDS wants:  128 image rows (the head-dim index d) x 8 chunks of 8 tile rows.
+//
+//   chunk c = 4*kt + 2*ss + g, element j   <->   tile row 32*(j>>2) + 16*g + 4*(j&3) + ss + 2*kt
+//
+// which is exactly the order in which lane group g holds the 8 contraction values of
+// k-step ss of sub-tile kt in an accumulator (acc_tile_row).  Inside the image, chunks
+// are stored chunk-major in groups of 16 image rows:
+//
+//   byte offset(d, c) = (d >> 4) * 2048 + c * 256 + (d & 15) * 16
+//
+// so the 16 lanes that are served together (16 consecutive d, same c) read 256
+// contiguous bytes: all 64 banks, no padding.  The image is contiguous in global
+// memory and in LDS, so the direct loads are plain 1 KB copies.
+constexpr int IMG_ELEMS = 128 * 64;          // 16384 bytes
+constexpr int IMG_BYTES = IMG_ELEMS * 2;
+
+// position (chunk * 8 + element) of tile row `row` (0..63) inside an image row
+__host__ __device__ __forceinline__ int image_pos(int row) {
+  const int kt = (row >> 1) & 1, ss = row & 1, g = (row >> 4) & 1, j = 4 * (row >> 5) + ((row >> 2) & 3);
+  return 8 * (4 * kt + 2 * ss + g) + j;
+}
+
+__device__ __forceinline__ void load_image_async(bf16* lds_img, const bf16* img, int wave, int lane) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int off = ((4 * j + wave) * 64 + lane) * 8;
+    __builtin_amdgcn_global_load_lds((global_void_ptr)(img + off), (lds_void_ptr)(lds_img + (4 * j + wave) * 512), 16,
+                                     0, 0);
+  }
+}
+
+// Per-lane element offset of the A operand read from an image: MFMA row i <-> d = 32*dt + i.
+// Add dt*2048 + (4*kt + 2*ss)*128 elements.
+__device__ __forceinline__ int image_frag_base(int g, int i) { return (i >> 4) * 1024 + (i & 15) * 8 + g * 128; }
+
+__device__ __forceinline__ bf16x8 image_frag(const bf16* img, int base, int dt, int ss, int kt) {
+  return *reinterpret_cast<const bf16x8*>(img + base + dt * 2048 + (4 * kt + 2 * ss) * 128);
+}
+
+}  // namespace tile128
+
+// O += A . B with the accumulator pinned in AccVGPRs.  The hot loops keep their large,
+// MFMA-only accumulators there so that the 256 architectural VGPRs stay free for values
+// the vector ALUs touch.  The compiler does not see an MFMA here: code that reads such an
+// accumulator with vector instructions must first let the matrix pipe drain (mfma_drain).
+__device__ __forceinline__ void mfma32_acc(f32x16& c, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+
+// Swap of the two wavefront halves through v_permlane32_swap: returns, in every lane,
+// op(x of this lane, x of the lane 32 away).
+__device__ __forceinline__ float half_swap_max(float x) {
+  const unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+  const unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}

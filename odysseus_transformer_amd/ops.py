@@ -55,9 +55,11 @@ def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=No
         out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    ws_bytes = _lib.load().ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     _lib.call("ody_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
               B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
-              scale, int(causal), _dt(q), _stream())
+              scale, int(causal), _dt(q), ws.data_ptr() if ws_bytes else 0, ws_bytes, _stream())
     return out, lse
 
 
@@ -75,7 +77,7 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     dv = torch.empty_like(v) if dv is None else dv
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     lib = _lib.load()
-    ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Hq)
+    ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")

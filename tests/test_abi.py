@@ -37,15 +37,15 @@ def test_validation_returns_codes_without_a_gpu():
         _lib.call("ody_gemm", 0, 0, 0, 0, 0, 8, 8, 8, 8, 8, 8, 0, 0, 0)
     assert e.value.code == -4 and "NULL" in e.value.msg
     with pytest.raises(_lib.OdysseusHipError) as e:
-        _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 3, 2, 128, *([128] * 12), 1.0, 1, 0, 0)
+        _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 3, 2, 128, *([128] * 12), 1.0, 1, 0, 0, 0, 0)
     assert e.value.code == -1 and "multiple" in e.value.msg
     with pytest.raises(_lib.OdysseusHipError) as e:
-        _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 2, 2, 96, *([128] * 12), 1.0, 1, 0, 0)
+        _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 2, 2, 96, *([128] * 12), 1.0, 1, 0, 0, 0, 0)
     assert e.value.code == -2
     with pytest.raises(_lib.OdysseusHipError) as e:
         _lib.call("ody_rmsnorm_fwd", 16, 16, 16, 0, 4, 7, 1e-6, 0, 0)
     assert e.value.code == -2
-    assert lib.ody_attn_bwd_workspace_bytes(1, 1000, 4) == 16128
+    assert lib.ody_attn_bwd_workspace_bytes(1, 1000, 1000, 4, 4, 64, 0) == 16128
     assert lib.ody_rmsnorm_bwd_partials(100) == 100 and lib.ody_rmsnorm_bwd_partials(100000) == 512
 
 
