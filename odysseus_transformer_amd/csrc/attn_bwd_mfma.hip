@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnParams p) 
   TileRegs<BQ, D> qr, dor;
   float lreg = 0.f, dreg = 0.f;
   auto gload = [&](int it) {
-    const int hg = it / ntq, i0 = i_begin + (it % ntq) * BQ, h = hk * p.group + hg;
+    const int hg = it / ntq, i0 = i_begin + (ntq - 1 - it % ntq) * BQ, h = hk * p.group + hg;
     const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
     const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
     qr.load(qp, p.sq.l, i0, p.Lq, tid);
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnParams p) 
 
   for (int it = 0; it < total; it++) {
     const int buf = it & 1;
-    const int i0 = i_begin + (it % ntq) * BQ;
+    const int i0 = i_begin + (ntq - 1 - it % ntq) * BQ;   // last query tile first: the key blocks running on an XCD then read the same Q / dO tiles together
     if (it + 1 < total) gload(it + 1);
     const bf16* Qb = Qs + buf * BQ * P;
     const bf16* Ob = Os + buf * BQ * P;
@@ -363,6 +363,24 @@ int launch(const AttnParams& p, hipStream_t st) {
 }
 
 }  // namespace
+
+// the dK/dV kernel alone (head_dim 128), for the launcher that pairs it with the dQ kernel of attn_bwd_pipe.hip
+int ody_launch_attn_bwd_dkdv_mfma(const AttnParams& p, hipStream_t st) {
+  constexpr int D = 128;
+  constexpr size_t smem_kv = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16) + 2 * 2 * 64 * sizeof(float);
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess) {
+      ody_set_error("attn_bwd: hipFuncSetAttribute failed");
+      return ODY_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  dim3 gk(((p.Lk + 127) / 128) * p.Hkv * p.B);
+  ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
+  return ody_check_launch("attn_bwd_dkdv");
+}
 
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st) {
   if (D == 128) return launch<128>(p, st);

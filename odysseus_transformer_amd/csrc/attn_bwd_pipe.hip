@@ -1,23 +1,17 @@
-// Flash-attention backward, head_dim 128, bf16, on the tile machinery of attn_tile.h:
-// direct global->LDS loads, 16-byte LDS reads only (operands that are contracted over
-// their row index come from the transposed images a pre-pass writes), fenced slots that
-// keep LDS operand prefetch, MFMAs and vector work interleaved.
+// Flash-attention backward, head_dim 128, bf16: the dQ kernel on the tile machinery of
+// attn_tile.h -- direct global->LDS loads into a three-deep ring, 16-byte LDS reads only
+// (K^T comes from the transposed images a pre-pass writes), fenced slots that keep LDS
+// operand prefetch and MFMAs interleaved.  Query-stationary, 8 wavefronts x 32 queries
+// (two wavefronts per SIMD overlap each other's matrix and vector phases), lane = query
+// column, so lse and delta are per-lane scalars:
 //
-// Two kernels, no atomics, deterministic (same split as attn_bwd_mfma.hip):
-//
-//  dQ kernel (query-stationary; 4 wavefronts x 64 queries, lane = query column)
 //      S^T = K Q^T            A: K rows (LDS)        B: Q^T (registers)
 //      dP^T = V dO^T          A: V rows (LDS)        B: dO^T (registers)
-//      dS^T = exp2(S^T c - lse) * (dP^T - delta)     per-lane lse / delta
+//      dS^T = exp2(S^T c - lse) * (dP^T - delta)
 //      dQ^T += K^T dS^T       A: K^T image (LDS)     B: dS^T = accumulator layout
 //
-//  dK/dV kernel (key-stationary; 4 wavefronts x 32 keys, lane = key column; loops over
-//  the query heads of the group and over 64-query tiles)
-//      S = Q K^T              A: Q rows (LDS)        B: K^T (registers)
-//      dP = dO V^T            A: dO rows (LDS)       B: V^T (registers)
-//      P = exp2(S c - lse), dS = P * (dP - delta)    lse / delta staged in LDS in accumulator order
-//      dV^T += dO^T P         A: dO^T image (LDS)    B: P
-//      dK^T += Q^T dS         A: Q^T image (LDS)     B: dS
+// The dK/dV half of the backward is the key-stationary kernel of attn_bwd_mfma.hip.  No
+// atomics anywhere: both kernels recompute S, and each owns its outputs.
 #include <type_traits>
 #include "attn_params.h"
 #include "attn_tile.h"
@@ -28,19 +22,11 @@ using namespace tile128;
 
 constexpr int D = 128, KS = D / 16, DT = D / 32;
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
-#ifdef ODY_DEBUG_CYCLES
-__device__ long long ody_dbg_bwd[16];
-#define DBG_T(v) const long long v = __builtin_amdgcn_s_memtime()
-#define DBG_ACC(slot, a, b) dbg[slot] += (b) - (a)
-#else
-#define DBG_T(v)
-#define DBG_ACC(slot, a, b)
-#endif
 
 // ---------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------
-constexpr int DQ_QT = 2, DQ_WAVES = 4, DQ_BM = 32 * DQ_QT * DQ_WAVES, DQ_THREADS = 64 * DQ_WAVES;
+constexpr int DQ_QT = 1, DQ_WAVES = 8, DQ_BM = 32 * DQ_QT * DQ_WAVES, DQ_THREADS = 64 * DQ_WAVES;
 
 __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const AttnParams p,
                                                                        const bf16* __restrict__ kimg) {
@@ -73,8 +59,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 
   auto load_stage = [&](bf16* st, int t) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int grp = 4 * j + wave;
+    for (int j = 0; j < 16 / DQ_WAVES; j++) {
+      const int grp = DQ_WAVES * j + wave;
       int row = t * BN + 4 * grp + (lane & 3);
       row = row < p.Lk ? row : p.Lk - 1;
       const int col = 8 * (lane >> 2);
@@ -123,13 +109,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 #pragma unroll
       for (int r = 0; r < 16; r++) dq[qt][dt][r] = 0.f;
 
-#ifdef ODY_DEBUG_CYCLES
-  long long dbg[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#endif
   // one 32-key sub-tile x 64 queries: 32 MFMAs for S^T and dP^T, the vector work, 16 MFMAs for
   // dQ^T; every LDS operand fragment feeds two MFMAs
   auto sub_tile = [&](const bf16* st, int t, int kt, bool masked) {
-    DBG_T(t0);
     const bf16* Kt = st + kt * 16;
     const bf16* Vt = st + TILE_ELEMS + kt * 16;
     const bf16* Ki = st + 2 * TILE_ELEMS + kt * 512;
@@ -160,7 +142,6 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
       }
       FENCE();
     }
-    DBG_T(t1);
     bf16x8 ifr[PF];
 #pragma unroll
     for (int n = 0; n < PF; n++) ifr[n] = image_frag(Ki, ibase, n & 3, n >> 2, 0);
@@ -180,7 +161,6 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
         dsf[qt][r >> 3][r & 7] = (bf16)(pr * (dp[qt][r] - delta[qt]));
       }
     FENCE();
-    DBG_T(t2);
 #pragma unroll
     for (int n = 0; n < 8; n++) {
       const int dt = n & 3, ss = n >> 2;
@@ -189,29 +169,23 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
       if (n + PF < 8) ifr[n % PF] = image_frag(Ki, ibase, (n + PF) & 3, (n + PF) >> 2, 0);
       FENCE();
     }
-    DBG_T(t3);
-    DBG_ACC(0, t0, t1); DBG_ACC(1, t1, t2); DBG_ACC(2, t2, t3); DBG_ACC(3, 0, 1);
   };
 
   for (int t = 0; t < ntiles; t++) {
-    DBG_T(ts0);
-    // stage t landed (the 12 loads of stage t+1 may still be in flight), everyone done with stage t-1
-    if (t + 1 < ntiles) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    // stage t landed (the loads of stage t+1 may still be in flight), everyone done with stage t-1
+    if (t + 1 < ntiles) {
+      if (DQ_WAVES == 8) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    }
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (t + 2 < ntiles) load_stage(ring + ((t + 2) % 3) * STAGE, t + 2);
     const bf16* st = ring + (t % 3) * STAGE;
-    DBG_T(ts1);
-    DBG_ACC(4, ts0, ts1);
     if (p.causal && t * BN > wq0 + 32 * QT - 1 + p.off) continue;   // every key of the tile is after this wavefront's queries
 #pragma unroll 1
     for (int kt = 0; kt < 2; kt++) sub_tile(st, t, kt, t >= n_full);
   }
 
-#ifdef ODY_DEBUG_CYCLES
-  if (blockIdx.x == 0 && lane == 0 && wave == 0)
-    for (int k = 0; k < 5; k++) ody_dbg_bwd[k] = dbg[k];
-#endif
 #pragma unroll
   for (int qt = 0; qt < QT; qt++) {
     const int qi = wq0 + 32 * qt + i;
@@ -232,255 +206,32 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   }
 }
 
-// ---------------------------------------------------------------------------------
-// dK / dV
-// ---------------------------------------------------------------------------------
-constexpr int KV_BN = 128, KV_BQ = 64;
-
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_pipe_kernel(const AttnParams p, const bf16* __restrict__ qimg,
-                                                                 const bf16* __restrict__ doimg) {
-  constexpr int STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + 2 * 64 * 2;   // Q, dO tiles; Q^T, dO^T images; lse, delta (fp32)
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][STAGE]
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
-  const BlockCoord bc = ody_block_coord(p.Hkv, p.B);   // rank 0 = first key block = most query tiles
-  const int hk = bc.h, b = bc.b;
-  const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
-  const bf16* kp = static_cast<const bf16*>(p.k) + b * p.sk.b + hk * p.sk.h;
-  const bf16* vp = static_cast<const bf16*>(p.v) + b * p.sv.b + hk * p.sv.h;
-  const int q_tiles = (p.Lq + KV_BQ - 1) / KV_BQ;
-
-  bf16x8 kf[KS], vf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ks++) {
-    if (key < p.Lk) {
-      kf[ks] = *reinterpret_cast<const bf16x8*>(kp + (int64_t)key * p.sk.l + 16 * ks + 8 * g);
-      vf[ks] = *reinterpret_cast<const bf16x8*>(vp + (int64_t)key * p.sv.l + 16 * ks + 8 * g);
-    } else {
-      kf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      vf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-  }
-  f32x16 dk[DT], dv[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) dk[dt][r] = dv[dt][r] = 0.f;
-
-  int t_begin = p.causal ? max(0, n0 - p.off) / KV_BQ : 0;   // first query tile that sees a key of this block
-  const int ntq = max(0, q_tiles - t_begin);
-  const int total = ntq * p.group;   // flattened (head of the group, query tile)
-  // query tiles from t_plain on need no causal mask for any key of the block; the ragged last
-  // query tile needs none either (its missing rows carry lse = +inf)
-  const int t_plain = p.causal ? (n0 + KV_BN - 1 - p.off + KV_BQ - 1) / KV_BQ : 0;
-
-  const float c2 = p.scale_log2e;
-  const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
-
-  auto load_stage = [&](bf16* st, int it) {
-    const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
-    const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
-    const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
-    const bf16* qi_ = qimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
-    const bf16* doi = doimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int grp = 4 * j + wave;
-      int row = t * KV_BQ + 4 * grp + (lane & 3);
-      row = row < p.Lq ? row : p.Lq - 1;
-      const int col = 8 * (lane >> 2);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (int64_t)row * p.sq.l + col),
-                                       (lds_void_ptr)(st + grp * GROUP_ELEMS), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(dop + (int64_t)row * p.sdo.l + col),
-                                       (lds_void_ptr)(st + TILE_ELEMS + grp * GROUP_ELEMS), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(qi_ + (grp * 64 + lane) * 8),
-                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + grp * 512), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(doi + (grp * 64 + lane) * 8),
-                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + IMG_ELEMS + grp * 512), 16, 0, 0);
-    }
-  };
-  // lse (as lse*log2e, +inf for rows that must give P = 0) and delta of the 64 queries of a tile,
-  // in accumulator order: position 32*mt + 16*g + r  <->  query acc_tile_row(r, g, mt)
-  float lreg = 0.f, dreg = 0.f;
-  auto load_stats = [&](int it) {
-    if (tid < 64) {
-      const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
-      const int mt = tid >> 5, gg = (tid >> 4) & 1, r = tid & 15;
-      const int qi = t * KV_BQ + acc_tile_row(r, gg, mt);
-      const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
-      float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
-      if (l == -INFINITY) l = INFINITY;
-      lreg = l * ODY_LOG2E;
-      dreg = (qi < p.Lq) ? p.delta[ri] : 0.f;
-    }
-  };
-  auto store_stats = [&](bf16* st) {
-    if (tid < 64) {
-      float* f = reinterpret_cast<float*>(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS);
-      f[tid] = lreg;
-      f[64 + tid] = dreg;
-    }
-  };
-
-  if (total > 0) {
-    load_stage(ring, 0);
-    load_stats(0);
-    store_stats(ring);
-  }
-
-  auto sub_tile = [&](const bf16* st, int t, int mt, auto masked) {
-    constexpr bool MASK = decltype(masked)::value;
-    const bf16* Qt = st;
-    const bf16* Ot = st + TILE_ELEMS;
-    const bf16* Qi = st + 2 * TILE_ELEMS;
-    const bf16* Oi = Qi + IMG_ELEMS;
-    const float* Ls = reinterpret_cast<const float*>(Oi + IMG_ELEMS) + 32 * mt + 16 * g;
-    const float* Ds = Ls + 64;
-    constexpr int PF = 3;
-    bf16x8 qfr[PF], ofr[PF];
-#pragma unroll
-    for (int n = 0; n < PF; n++) {
-      qfr[n] = row_frag(Qt, rbase, n, mt);
-      ofr[n] = row_frag(Ot, rbase, n, mt);
-    }
-    f32x16 s, dp;
-    FENCE();
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      if (ks == 0) {
-        s = mfma32(qfr[0], kf[0], f32x16{0});
-        dp = mfma32(ofr[0], vf[0], f32x16{0});
-      } else {
-        s = mfma32(qfr[ks % PF], kf[ks], s);
-        dp = mfma32(ofr[ks % PF], vf[ks], dp);
-      }
-      if (ks + PF < KS) {
-        qfr[ks % PF] = row_frag(Qt, rbase, ks + PF, mt);
-        ofr[ks % PF] = row_frag(Ot, rbase, ks + PF, mt);
-      }
-      FENCE();
-    }
-    bf16x8 oif[PF], qif[PF];
-#pragma unroll
-    for (int n = 0; n < PF; n++) {
-      oif[n] = image_frag(Oi, ibase, n & 3, n >> 2, mt);
-      qif[n] = image_frag(Qi, ibase, n & 3, n >> 2, mt);
-    }
-    bf16x8 pf[2], dsf[2];
-#pragma unroll
-    for (int a = 0; a < 4; a++) {
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(Ls + 4 * a);
-      const f32x4 d4 = *reinterpret_cast<const f32x4*>(Ds + 4 * a);
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        const int r = 4 * a + e;
-        float pr = ody_exp2(fmaf(s[r], c2, -l4[e]));
-        if constexpr (MASK)
-          if (key > t * KV_BQ + acc_tile_row(r, g, mt) + p.off) pr = 0.f;
-        pf[r >> 3][r & 7] = (bf16)pr;
-        dsf[r >> 3][r & 7] = (bf16)(pr * (dp[r] - d4[e]));
-      }
-    }
-    FENCE();
-#pragma unroll
-    for (int n = 0; n < 8; n++) {
-      const int dt = n & 3, ss = n >> 2;
-      dv[dt] = mfma32(oif[n % PF], pf[ss], dv[dt]);
-      dk[dt] = mfma32(qif[n % PF], dsf[ss], dk[dt]);
-      if (n + PF < 8) {
-        oif[n % PF] = image_frag(Oi, ibase, (n + PF) & 3, (n + PF) >> 2, mt);
-        qif[n % PF] = image_frag(Qi, ibase, (n + PF) & 3, (n + PF) >> 2, mt);
-      }
-      FENCE();
-    }
-  };
-
-  for (int it = 0; it < total; it++) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    const int t = q_tiles - 1 - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
-                                              // Q / dO tiles at the same time and share them through L2
-    if (it + 1 < total) {
-      load_stage(ring + ((it + 1) & 1) * STAGE, it + 1);
-      load_stats(it + 1);
-    }
-    const bf16* st = ring + (it & 1) * STAGE;
-    // every query of the tile is before every key of this wavefront: nothing to do
-    const bool dead = p.causal && (t * KV_BQ + KV_BQ - 1 + p.off < wn0);
-    if (!dead) {
-      if (t >= t_plain) {
-        sub_tile(st, t, 0, std::false_type{});
-        sub_tile(st, t, 1, std::false_type{});
-      } else {
-        sub_tile(st, t, 0, std::true_type{});
-        sub_tile(st, t, 1, std::true_type{});
-      }
-    }
-    if (it + 1 < total) store_stats(ring + ((it + 1) & 1) * STAGE);
-  }
-
-  if (key < p.Lk) {
-    bf16* dkp = static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l;
-    bf16* dvp = static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l;
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-      for (int a = 0; a < 4; a++) {
-        bf16x4 wk, wv;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          wk[e] = (bf16)(dk[dt][4 * a + e] * p.scale);
-          wv[e] = (bf16)dv[dt][4 * a + e];
-        }
-        *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = wk;
-        *reinterpret_cast<bf16x4*>(dvp + 32 * dt + 8 * a + 4 * g) = wv;
-      }
-  }
-}
-
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 }  // namespace
 
-// workspace after delta: [K^T images | Q^T images | dO^T images]
+// workspace after delta: the transposed images of K
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
-  return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq));
+  (void)Lq; (void)Hq;
+  return align256(ody_attn_images_bytes(B, Lk, Hkv));
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem_q = (size_t)3 * (2 * TILE_ELEMS + IMG_ELEMS) * sizeof(bf16);
-  constexpr size_t smem_kv = (size_t)2 * (2 * TILE_ELEMS + 2 * IMG_ELEMS + 2 * 64 * 2) * sizeof(bf16);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q) != hipSuccess) {
       ody_set_error("attn_bwd: hipFuncSetAttribute failed");
       return ODY_ERR_LAUNCH;
     }
     attr_set = true;
   }
-  char* ws = static_cast<char*>(workspace);
-  bf16* kimg = reinterpret_cast<bf16*>(ws);
-  bf16* qimg = reinterpret_cast<bf16*>(ws + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)));
-  bf16* doimg = reinterpret_cast<bf16*>(reinterpret_cast<char*>(qimg) + align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
+  bf16* kimg = static_cast<bf16*>(workspace);
   int rc;
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
-  if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
-  if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
-  dim3 gk(((p.Lk + KV_BN - 1) / KV_BN) * p.Hkv * p.B);
-  ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel, gk, dim3(256), smem_kv, p, qimg, doimg);
-  if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
+  if ((rc = ody_launch_attn_bwd_dkdv_mfma(p, st))) return rc;
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");
 }
-
-#ifdef ODY_DEBUG_CYCLES
-extern "C" int ody_debug_cycles_bwd(long long* out) {
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(ody_dbg_bwd), sizeof(long long) * 16) == hipSuccess ? 0 : -1;
-}
-#endif

@@ -17,7 +17,6 @@
 // written as 32 fenced slots {prefetch an operand for a later MFMA, one MFMA, a slice of
 // vector work}.  K runs ahead of V: the K ring holds three 64-key tiles, the V ring two
 // images, both filled by direct global->LDS loads (no staging registers, no LDS stores).
-// O lives in AccVGPRs (mfma32_acc); S, P, Q and the operand fragments in VGPRs.
 //
 // The softmax reference of a query is FIXED by its first 32 keys; exp2 of later scores
 // uses it as long as they exceed it by less than 2^64 (fp32 sums and bf16 P have the
@@ -40,14 +39,6 @@ constexpr float LAZY_LOG2 = 64.0f;
 // nothing may be moved across a fence by the instruction scheduler
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
-#ifdef ODY_DEBUG_CYCLES
-__device__ long long ody_dbg_cycles[16];
-#define DBG_T(v) const long long v = __builtin_amdgcn_s_memtime()
-#define DBG_ACC(slot, a, b) dbg[slot] += (b) - (a)
-#else
-#define DBG_T(v)
-#define DBG_ACC(slot, a, b)
-#endif
 
 struct SoftState {
   float ref_c;   // reference * scale*log2e (0 while no key has been seen)
@@ -117,10 +108,6 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
   const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
 
   f32x16 sA[QT], sB[QT];
-#ifdef ODY_DEBUG_CYCLES
-  long long dbg[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  const long long dbg_start = __builtin_amdgcn_s_memtime();
-#endif
 
   // per-thread element offsets of the 4 direct loads of a K tile (rows 4*grp + (lane & 3), chunk lane >> 2)
   unsigned koff[4];
@@ -205,9 +192,7 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
   //   slots  0..15: S(j+1) += K Q^T   with   P(j) elements 0..23
   //   slots 16..31: O += V(j) P(j)    with   P(j) elements 24..31, row max of S(j+1)
   auto step = [&](int j, f32x16 (&s_cur)[QT], f32x16 (&s_nxt)[QT], float (&mx)[QT]) {
-    DBG_T(t0);
     if ((j & 1) == 0) sync_and_prefetch(j >> 1);
-    DBG_T(t1);
     const int kt = j & 1, ktn = (j + 1) & 1;
     const bf16* Kt = Kring + (((j + 1) >> 1) % 3) * TILE_ELEMS;
     const bf16* Vt = Vring + ((j >> 1) & 1) * IMG_ELEMS;
@@ -227,7 +212,6 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
       for (int e = (3 * n) >> 1; e < (3 * (n + 1)) >> 1; e++) prob1(s_cur, pb, e);
       FENCE();
     }
-    DBG_T(t2);
     bf16x8 vfr[VPF];
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) mx[qt] = -INFINITY;
@@ -248,8 +232,6 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) mx[qt] = half_swap_max(mx[qt]);
     check_window(mx);
-    DBG_T(t3);
-    DBG_ACC(0, t0, t1); DBG_ACC(1, t1, t2); DBG_ACC(2, t2, t3); DBG_ACC(4, 0, 1);
   };
   // The plain (unpipelined) treatment of sub-tile j whose S and row maxima are at hand: moves
   // the reference if needed, then P and O += V P.  Used where the pipeline does not reach:
@@ -299,12 +281,6 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
     }
   }
 
-#ifdef ODY_DEBUG_CYCLES
-  if (blockIdx.x == 0 && lane == 0 && wave == 0) {
-    for (int k = 0; k < 5; k++) ody_dbg_cycles[k] = dbg[k];
-    ody_dbg_cycles[5] = __builtin_amdgcn_s_memtime() - dbg_start;
-  }
-#endif
   // ---- epilogue ----------------------------------------------------------------------
   if (bail && lane == 0) atomicOr(bail_flags + ((int64_t)b * p.Hq + h) * nqb + qblk, 1);
   bf16* op = static_cast<bf16*>(p.out) + b * p.so.b + h * p.so.h;
@@ -362,8 +338,3 @@ int ody_launch_attn_fwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   return ody_launch_attn_fwd_mfma_flagged(p, flags, BM, st);
 }
 
-#ifdef ODY_DEBUG_CYCLES
-extern "C" int ody_debug_cycles(long long* out) {
-  return hipMemcpyFromSymbol(out, HIP_SYMBOL(ody_dbg_cycles), sizeof(long long) * 16) == hipSuccess ? 0 : -1;
-}
-#endif

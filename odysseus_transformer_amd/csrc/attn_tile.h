@@ -1,6 +1,6 @@
-// LDS tiles of the head_dim-128 attention kernels: 64 rows x 128 bf16, filled by
-// direct global->LDS loads and read both row-wise (16-byte reads) and transposed
-// (ds_read_b64_tr_b16) without bank conflicts, with purely additive addressing.
+// LDS tiles of the head_dim-128 attention kernels: 64 rows x 128 bf16, filled by direct
+// global->LDS loads and read with 16-byte reads, without bank conflicts and with purely
+// additive addressing.
 //
 // A direct load (global_load_lds_dwordx4) makes the 64 lanes of a wavefront write
 // 64 consecutive 16-byte slots of LDS, each lane fetching from its own global
@@ -11,14 +11,10 @@
 //
 //     offset(row, col) = (row >> 2) * 520 + (col >> 3) * 32 + (row & 3) * 8 + (col & 7)
 //
-//  * row-wise operand: the 16 lanes that are served together read the same chunk
-//    of rows 4*i + b (i = 0..15, b fixed): their addresses are 1040 bytes apart,
-//    i.e. 4 banks apart -> 64 distinct banks;
-//  * transposed operand: one 16-lane block reads 4 rows of 4 consecutive groups
-//    (same b) x 2 chunks x 2 halves: banks 4t + 16x + 2y (+0/1), all distinct.
-//
-// To make both patterns line up, row rho (0..31) of a 32-row MFMA operand of
-// sub-tile kt (0/1) is tile row  4*(rho & 15) + (rho >> 4) + 2*kt.
+// The 16 lanes that are served together read the same chunk of rows 4*i + b
+// (i = 0..15, b fixed): their addresses are 1040 bytes apart, i.e. 4 banks apart ->
+// 64 distinct banks.  For that, row rho (0..31) of a 32-row MFMA operand of sub-tile
+// kt (0/1) is tile row  4*(rho & 15) + (rho >> 4) + 2*kt.
 #pragma once
 #include "ody_common.h"
 
@@ -62,19 +58,6 @@ __device__ __forceinline__ int row_frag_base(int g, int i) { return (i & 15) * G
 
 __device__ __forceinline__ bf16x8 row_frag(const bf16* tile, int base, int ks, int kt) {
   return *reinterpret_cast<const bf16x8*>(tile + base + ks * 64 + kt * 16);
-}
-
-// Per-lane element offset of the transposed operand: this lane supplies the address of
-// 4 consecutive columns of one row; after the transpose read the lane holds column
-// 32*dt + i of the rows that k-step ss of sub-tile kt contracts over (first half: rows
-// of groups 4g..4g+3, second half: +8 groups).  Add dt*128 + (ss + 2*kt)*8 (+ 8 groups).
-__device__ __forceinline__ int tr_frag_base(int g, int i) {
-  return (4 * g + ((i & 15) >> 2)) * GROUP_ELEMS + (2 * (i >> 4) + ((i & 3) >> 1)) * 32 + 4 * (i & 1);
-}
-
-__device__ __forceinline__ bf16x8 tr_frag(const bf16* tile, int base, int dt, int ss, int kt) {
-  const bf16* p = tile + base + dt * 128 + (ss + 2 * kt) * 8;
-  return concat4(lds_read_tr16(p), lds_read_tr16(p + 8 * GROUP_ELEMS));
 }
 
 // ---------------------------------------------------------------------------------
@@ -123,15 +106,6 @@ __device__ __forceinline__ bf16x8 image_frag(const bf16* img, int base, int dt, 
 }
 
 }  // namespace tile128
-
-// O += A . B with the accumulator pinned in AccVGPRs.  The hot loops keep their large,
-// MFMA-only accumulators there so that the 256 architectural VGPRs stay free for values
-// the vector ALUs touch.  The compiler does not see an MFMA here: code that reads such an
-// accumulator with vector instructions must first let the matrix pipe drain (mfma_drain).
-__device__ __forceinline__ void mfma32_acc(f32x16& c, bf16x8 a, bf16x8 b) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 // Swap of the two wavefront halves through v_permlane32_swap: returns, in every lane,
 // op(x of this lane, x of the lane 32 away).

@@ -101,6 +101,28 @@ def test_attention_row_properties(dev):
         assert rel_err(o[0, rows, h], ref_o) <= TOL_BF16
 
 
+def test_attention_scores_beyond_the_reference_window(dev):
+    """The head_dim-128 forward fixes its softmax reference from the first keys and hands a
+    query block whose later scores exceed it by more than 2^64 to the online-rescaling
+    kernel: the results must be right on both sides of that switch."""
+    from odysseus_transformer_amd import ops
+    B, L, H, D = 1, 700, 2, 128
+    q, k, v, do = _inputs(B, L, L, H, H, D, torch.bfloat16, seed=29)
+    # head 0: early keys score about -90, a run of late keys about +90 (in units of log 2: +-130)
+    q[:, :, 0] = 2.0
+    k[:, :, 0] = -4.0
+    k[:, 500:520, 0] = 4.0
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=True)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float())
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=True)
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    assert rel_err(o, o_ref) <= TOL_BF16
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True)
+    assert rel_err(dq, dq_ref) <= TOL_BF16 and rel_err(dk, dk_ref) <= TOL_BF16 and rel_err(dv, dv_ref) <= TOL_BF16
+
+
 def test_attention_errors(dev):
     from odysseus_transformer_amd import ops
     from odysseus_transformer_amd._lib import OdysseusHipError
