@@ -52,6 +52,17 @@ def time_gpu(fn, iters, warmup):
     return (time.perf_counter() - t0) / iters
 
 
+def measured_traffic():
+    """HBM bytes per launch of the attention kernels at this workload, as measured with the
+    FETCH_SIZE / WRITE_SIZE counters and recorded (as a JSON block) in the profile summary."""
+    import re
+    f = ROOT / "profiles" / "attention_L32768_hbm_traffic.md"
+    if not f.exists():
+        return {}
+    m = re.search(r"```json\s*(\{.*?\})\s*```", f.read_text(), re.S)
+    return json.loads(m.group(1)) if m else {}
+
+
 def cpu_baseline():
     """The oracle (plain PyTorch, fp32) on the host cores: causal attention fwd+bwd at
     4 heads x 128, L = 8192 -- 1/16 of the FLOPs of one benchmark step."""
@@ -77,9 +88,13 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-layer", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain device copy of the packed qkv buffer (100 MiB read + 100 MiB "
+                         "written): the known-size kernel that calibrates the HBM byte counters of a "
+                         "rocprofv3 --pmc run of this script")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU's share of the layer on ONE GPU; collectives and multi-GPU runs are "
@@ -115,6 +130,8 @@ def main():
 
     for _ in range(a.warmup):
         step()
+    if a.copy_probe:
+        dqkv.copy_(qkv)
     torch.cuda.synchronize()
     _lib.profile_enable(True)
     _lib.profile_collect()
@@ -139,10 +156,7 @@ def main():
     dom = max(algo, key=lambda n: prof[n][1] / prof[n][0])
     dom_avg = prof[dom][1] / prof[dom][0]
     achieved = algo[dom] / (dom_avg * 1e-3) / 1e12
-    traffic = None
-    tf = ROOT / "profiles" / "attn_hbm_traffic.json"
-    if tf.exists():
-        traffic = json.loads(tf.read_text()).get(dom)
+    traffic = measured_traffic().get(dom)
     value = (f_fwd + f_bwd) / sec / 1e12
 
     out = {

@@ -268,3 +268,22 @@ def test_decoder_layer_explicit_bwd_vs_autograd_and_hf_layer():
     out = layer(x, attention_mask=mask, position_ids=pos, position_embeddings=(cos, sin))
     out = out[0] if isinstance(out, tuple) else out
     assert torch.allclose(out, y2, atol=1e-5)      # HF's eager softmax runs in fp32
+
+
+# ------------------------------------------------------------------ the sampled checker used at full sizes
+@pytest.mark.parametrize("Hq,Hkv,Lq,Lk", [(4, 2, 300, 300), (2, 1, 130, 390)])
+def test_sampled_checker_accepts_the_oracle_and_rejects_mistakes(Hq, Hkv, Lq, Lk):
+    from sampled import edge_samples, sampled_checks
+    D = 32
+    q, do = randn((1, Lq, Hq, D), 90), randn((1, Lq, Hq, D), 91)
+    k, v = randn((1, Lk, Hkv, D), 92), randn((1, Lk, Hkv, D), 93)
+    o, lse = oracle.attention_fwd(q, k, v, causal=True)
+    dq, dk, dv = oracle.attention_bwd(q, k, v, o, lse, do, causal=True)
+    rows, cols = edge_samples(Lq, 5, 1), edge_samples(Lk, 5, 2)
+    args = [q[0], k[0], v[0], do[0], o[0], lse[0], dq[0], dk[0], dv[0]]
+    sampled_checks(*args, True, rows, cols)
+    for idx, bad in ((4, -o[0]), (6, dq[0] * 1.1), (7, dk[0].flip(0)), (8, dv[0] + 0.05 * dv[0].abs().max())):
+        wrong = list(args)
+        wrong[idx] = bad
+        with pytest.raises(AssertionError):
+            sampled_checks(*wrong, True, rows, cols)
