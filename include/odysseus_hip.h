@@ -67,7 +67,8 @@ int ody_profile_collect(char* out, size_t cap);
  * GQA: q head h reads kv head h / (Hq / Hkv).  causal != 0 masks key j for
  * query i when j > i + (Lk - Lq).  D in {64, 128}.
  * workspace: ody_attn_fwd_workspace_bytes(...) bytes, 256-byte aligned (the bf16
- * head_dim-128 kernel keeps a transposed copy of V there; 0 bytes = may be NULL).
+ * head_dim-128 kernel keeps a transposed copy of V and one int per 256-query block
+ * there; 0 bytes = may be NULL).
  */
 size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -88,7 +89,7 @@ int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* 
  * no atomics).  If accumulate_dq != 0 the kernel adds into dq (fp32 dq_accum
  * layout not needed: the add happens in fp32 before rounding once).
  * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
- * the bf16 head_dim-128 kernels the transposed copies of K, Q and dO).
+ * the bf16 head_dim-128 kernels a transposed copy of K).
  */
 size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,

@@ -233,6 +233,54 @@ class FlashAttnFunc(torch.autograd.Function):
         return dq, dk, dv, None, None
 
 
+class RingBlocksAttnFunc(torch.autograd.Function):
+    """One rank's inner loop of ring attention (entered at decoder/ring.py:30-37 in the reference):
+    the local queries against a sequence of K/V blocks as they would arrive over the ring.  Block
+    `causal_block` is the diagonal one (causally masked); every other block is fully visible.
+    Forward merges each block's (out, lse) into an fp32 running pair; backward runs the per-block
+    flash backward with the FINAL out / lse and accumulates dq over the blocks.
+
+    apply(q, causal_block, softmax_scale, *k_blocks, *v_blocks) -> (out, lse)."""
+
+    @staticmethod
+    def forward(ctx, q, causal_block, softmax_scale, *kv):
+        nb = len(kv) // 2
+        ks, vs = kv[:nb], kv[nb:]
+        B, L, H, D = q.shape
+        acc = torch.zeros((B, L, H, D), dtype=torch.float32, device=q.device)
+        lse = torch.full((B, H, L), float("-inf"), dtype=torch.float32, device=q.device)
+        for b in range(nb):
+            ob, lb = attn_fwd(q, ks[b], vs[b], causal=(b == causal_block), scale=softmax_scale)
+            lse_merge_(acc, lse, ob, lb)
+        out = acc.to(q.dtype)
+        ctx.save_for_backward(q, out, lse, *kv)
+        ctx.causal_block, ctx.softmax_scale = causal_block, softmax_scale
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, out, lse, *kv = ctx.saved_tensors
+        nb = len(kv) // 2
+        ks, vs = kv[:nb], kv[nb:]
+        if dout.stride(3) != 1:
+            dout = dout.contiguous()
+        dq = torch.empty_like(q)
+        dks, dvs = [], []
+        for b in range(nb):
+            _, dk, dv = attn_bwd(q, ks[b], vs[b], out, lse, dout, causal=(b == ctx.causal_block),
+                                 scale=ctx.softmax_scale, dq=dq, accumulate_dq=(b > 0))
+            dks.append(dk)
+            dvs.append(dv)
+        return (dq, None, None, *dks, *dvs)
+
+
+def ring_blocks_attn(q, k_blocks, v_blocks, causal_block: Optional[int] = 0, softmax_scale: Optional[float] = None):
+    """Functional form of RingBlocksAttnFunc; causal_block=None makes every block fully visible."""
+    cb = -1 if causal_block is None else int(causal_block)
+    return RingBlocksAttnFunc.apply(q, cb, softmax_scale, *k_blocks, *v_blocks)
+
+
 def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[float] = None, causal: bool = False,
                     return_lse: bool = False):
     """Signature of the routine the reference reaches at decoder/odysseus.py:256-263.

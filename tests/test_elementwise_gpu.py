@@ -142,3 +142,27 @@ def test_ring_step_equals_unsplit_attention(dev):
     assert rel_err(dq, dq_ref) <= TOL_BF16
     assert rel_err(torch.cat(dks[1:] + dks[:1], 1), dk_ref) <= TOL_BF16
     assert rel_err(torch.cat(dvs[1:] + dvs[:1], 1), dv_ref) <= TOL_BF16
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_ring_blocks_autograd_function(dtype, dev):
+    """ops.ring_blocks_attn (forward merge + backward over blocks under autograd) vs. the oracle's ring loop."""
+    from odysseus_transformer_amd import ops
+    B, Lq, H, Hkv, D, NB = 1, 200, 4, 2, 64, 3
+    tol = TOL_BF16 if dtype == torch.bfloat16 else 1e-4
+    q = randn((B, Lq, H, D), 71, dtype=dtype)
+    ks = [randn((B, Lq, Hkv, D), 72 + b, dtype=dtype) for b in range(NB)]
+    vs = [randn((B, Lq, Hkv, D), 82 + b, dtype=dtype) for b in range(NB)]
+    do = randn((B, Lq, H, D), 70, dtype=dtype)
+    f = lambda ts: [t.float() for t in ts]
+    o_ref, l_ref = oracle.ring_attention_fwd(q.float(), f(ks), f(vs), causal_block=1)
+    dq_ref, dk_ref, dv_ref = oracle.ring_attention_bwd(q.float(), f(ks), f(vs), o_ref, l_ref, do.float(), causal_block=1)
+    qg = q.to(dev).requires_grad_()
+    kg = [t.to(dev).requires_grad_() for t in ks]
+    vg = [t.to(dev).requires_grad_() for t in vs]
+    out, lse = ops.ring_blocks_attn(qg, kg, vg, causal_block=1)
+    out.backward(do.to(dev))
+    assert rel_err(out, o_ref) <= tol and torch.allclose(lse.cpu(), l_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    assert rel_err(qg.grad, dq_ref) <= tol
+    for b in range(NB):
+        assert rel_err(kg[b].grad, dk_ref[b]) <= tol and rel_err(vg[b].grad, dv_ref[b]) <= tol
