@@ -206,31 +206,246 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   }
 }
 
+// ---------------------------------------------------------------------------------
+// dK / dV
+// ---------------------------------------------------------------------------------
+// Key-stationary, 8 wavefronts x 32 keys (two wavefronts per SIMD), lane = key column.  K and V
+// rows stay in registers as B operands; 64-query tiles of Q and dO stream through a two-deep
+// ring as row tiles (A operands of S and dP) and as transposed images (A operands of dV^T and
+// dK^T); P and dS are accumulator tiles, which is the B-operand layout of the next product.
+//
+//      S  = Q K^T - lse/scale     the accumulator starts at -lse/scale, so P = exp2(S c)
+//      dP = dO V^T - delta        the accumulator starts at -delta
+//      dV^T += dO^T P             dK^T += Q^T (P o dP)
+constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 * KV_WAVES;
+constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + 2 * 64 * 2;   // Q, dO tiles; Q^T, dO^T images; 2 x 64 floats
+
+__global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
+                                                                         const bf16* __restrict__ qimg,
+                                                                         const bf16* __restrict__ doimg) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][KV_STAGE]
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
+  const BlockCoord bc = ody_block_coord(p.Hkv, p.B);   // rank 0 = first key block = most query tiles
+  const int hk = bc.h, b = bc.b;
+  const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
+  const int q_tiles = (p.Lq + KV_BQ - 1) / KV_BQ;
+
+  bf16x8 kf[KS], vf[KS];
+  {
+    const bf16* kp = static_cast<const bf16*>(p.k) + b * p.sk.b + hk * p.sk.h;
+    const bf16* vp = static_cast<const bf16*>(p.v) + b * p.sv.b + hk * p.sv.h;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if (key < p.Lk) {
+        kf[ks] = *reinterpret_cast<const bf16x8*>(kp + (int64_t)key * p.sk.l + 16 * ks + 8 * g);
+        vf[ks] = *reinterpret_cast<const bf16x8*>(vp + (int64_t)key * p.sv.l + 16 * ks + 8 * g);
+      } else {
+        kf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        vf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      }
+    }
+  }
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dk[dt][r] = dv[dt][r] = 0.f;
+
+  const int t_begin = p.causal ? max(0, n0 - p.off) / KV_BQ : 0;   // first query tile that sees a key of this block
+  const int ntq = max(0, q_tiles - t_begin);
+  const int total = ntq * p.group;   // flattened (head of the group, query tile)
+  const float c2 = p.scale_log2e, inv_scale = 1.0f / p.scale;
+  const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
+
+  auto load_stage = [&](bf16* st, int it) {
+    const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
+    const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
+    const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
+    const bf16* qi_ = qimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
+    const bf16* doi = doimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
+#pragma unroll
+    for (int j = 0; j < 16 / KV_WAVES; j++) {
+      const int grp = KV_WAVES * j + wave;
+      int row = t * KV_BQ + 4 * grp + (lane & 3);
+      row = row < p.Lq ? row : p.Lq - 1;
+      const int col = 8 * (lane >> 2);
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (int64_t)row * p.sq.l + col),
+                                       (lds_void_ptr)(st + grp * GROUP_ELEMS), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(dop + (int64_t)row * p.sdo.l + col),
+                                       (lds_void_ptr)(st + TILE_ELEMS + grp * GROUP_ELEMS), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(qi_ + (grp * 64 + lane) * 8),
+                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + grp * 512), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(doi + (grp * 64 + lane) * 8),
+                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + IMG_ELEMS + grp * 512), 16, 0, 0);
+    }
+  };
+  // the accumulator start values of the 64 queries of a tile, in accumulator order:
+  // position 32*mt + 16*g + r  <->  query acc_tile_row(r, g, mt).  -lse/scale (-inf for rows that
+  // must give P = 0: beyond Lq, or a query that saw no key) and -delta.
+  float lreg = 0.f, dreg = 0.f;
+  auto load_stats = [&](int it) {
+    if (tid < 64) {
+      const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
+      const int mt = tid >> 5, gg = (tid >> 4) & 1, r = tid & 15;
+      const int qi = t * KV_BQ + acc_tile_row(r, gg, mt);
+      const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
+      float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
+      if (l == -INFINITY) l = INFINITY;
+      lreg = -l * inv_scale;
+      dreg = (qi < p.Lq) ? -p.delta[ri] : 0.f;
+    }
+  };
+  auto store_stats = [&](bf16* st) {
+    if (tid < 64) {
+      float* f = reinterpret_cast<float*>(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS);
+      f[tid] = lreg;
+      f[64 + tid] = dreg;
+    }
+  };
+
+  if (total > 0) {
+    load_stage(ring, 0);
+    load_stats(0);
+    store_stats(ring);
+  }
+
+  // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
+  // work, 16 MFMAs for dV^T and dK^T
+  auto sub_tile = [&](const bf16* st, int t, int mt, bool masked) {
+    const bf16* Qt = st;
+    const bf16* Ot = st + TILE_ELEMS;
+    const bf16* Qi = st + 2 * TILE_ELEMS;
+    const bf16* Oi = Qi + IMG_ELEMS;
+    const float* Ls = reinterpret_cast<const float*>(Oi + IMG_ELEMS) + 32 * mt + 16 * g;
+    constexpr int PF = 2;
+    bf16x8 qfr[PF], ofr[PF];
+#pragma unroll
+    for (int n = 0; n < PF; n++) {
+      qfr[n] = row_frag(Qt, rbase, n, mt);
+      ofr[n] = row_frag(Ot, rbase, n, mt);
+    }
+    f32x16 s = *reinterpret_cast<const f32x16*>(Ls);
+    f32x16 dp = *reinterpret_cast<const f32x16*>(Ls + 64);
+    FENCE();
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      s = mfma32(qfr[ks % PF], kf[ks], s);
+      dp = mfma32(ofr[ks % PF], vf[ks], dp);
+      if (ks + PF < KS) {
+        qfr[ks % PF] = row_frag(Qt, rbase, ks + PF, mt);
+        ofr[ks % PF] = row_frag(Ot, rbase, ks + PF, mt);
+      }
+      FENCE();
+    }
+    bf16x8 oif[PF], qif[PF];
+#pragma unroll
+    for (int n = 0; n < PF; n++) {
+      oif[n] = image_frag(Oi, ibase, n & 3, n >> 2, mt);
+      qif[n] = image_frag(Qi, ibase, n & 3, n >> 2, mt);
+    }
+    if (masked) {
+      const int lim = key - p.off - t * KV_BQ;   // tile rows below lim come before this key
+#pragma unroll
+      for (int r = 0; r < 16; r++)
+        if (acc_tile_row(r, g, mt) < lim) s[r] = -INFINITY;
+    }
+    bf16x8 pf[2], dsf[2];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const float pr = ody_exp2(s[r] * c2);
+      pf[r >> 3][r & 7] = (bf16)pr;
+      dsf[r >> 3][r & 7] = (bf16)(pr * dp[r]);
+    }
+    FENCE();
+#pragma unroll
+    for (int n = 0; n < 8; n++) {
+      const int dt = n & 3, ss = n >> 2;
+      dv[dt] = mfma32(oif[n % PF], pf[ss], dv[dt]);
+      dk[dt] = mfma32(qif[n % PF], dsf[ss], dk[dt]);
+      if (n + PF < 8) {
+        oif[n % PF] = image_frag(Oi, ibase, (n + PF) & 3, (n + PF) >> 2, mt);
+        qif[n % PF] = image_frag(Qi, ibase, (n + PF) & 3, (n + PF) >> 2, mt);
+      }
+      FENCE();
+    }
+  };
+
+  for (int it = 0; it < total; it++) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int t = q_tiles - 1 - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
+                                              // Q / dO tiles at the same time and share them through L2
+    if (it + 1 < total) {
+      load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1);
+      load_stats(it + 1);
+    }
+    const bf16* st = ring + (it & 1) * KV_STAGE;
+    // every query of the tile is before every key of this wavefront: nothing to do
+    const bool dead = p.causal && (t * KV_BQ + KV_BQ - 1 + p.off < wn0);
+    if (!dead) {
+      const bool masked = p.causal && (t * KV_BQ + p.off < wn0 + 31);
+#pragma unroll 1
+      for (int mt = 0; mt < 2; mt++) sub_tile(st, t, mt, masked);
+    }
+    if (it + 1 < total) store_stats(ring + ((it + 1) & 1) * KV_STAGE);
+  }
+
+  if (key < p.Lk) {
+    bf16* dkp = static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l;
+    bf16* dvp = static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        bf16x4 wk, wv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          wk[e] = (bf16)(dk[dt][4 * a + e] * p.scale);
+          wv[e] = (bf16)dv[dt][4 * a + e];
+        }
+        *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = wk;
+        *reinterpret_cast<bf16x4*>(dvp + 32 * dt + 8 * a + 4 * g) = wv;
+      }
+  }
+}
+
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 }  // namespace
 
-// workspace after delta: the transposed images of K
+// workspace after delta: the transposed images of K, Q and dO
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
-  (void)Lq; (void)Hq;
-  return align256(ody_attn_images_bytes(B, Lk, Hkv));
+  return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq));
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem_q = (size_t)3 * (2 * TILE_ELEMS + IMG_ELEMS) * sizeof(bf16);
+  constexpr size_t smem_kv = (size_t)2 * KV_STAGE * sizeof(bf16);
   static bool attr_set = false;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q) != hipSuccess) {
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess) {
       ody_set_error("attn_bwd: hipFuncSetAttribute failed");
       return ODY_ERR_LAUNCH;
     }
     attr_set = true;
   }
-  bf16* kimg = static_cast<bf16*>(workspace);
+  unsigned char* w = static_cast<unsigned char*>(workspace);
+  bf16* kimg = reinterpret_cast<bf16*>(w);
+  bf16* qimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)));
+  bf16* doimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)) +
+                                        align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
   int rc;
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
-  if ((rc = ody_launch_attn_bwd_dkdv_mfma(p, st))) return rc;
+  if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
+  if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
+  dim3 gk(((p.Lk + KV_BN - 1) / KV_BN) * p.Hkv * p.B);
+  ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel, gk, dim3(KV_THREADS), smem_kv, p, qimg, doimg);
+  if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");
