@@ -220,13 +220,33 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 * KV_WAVES;
 constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + 2 * 64 * 2;   // Q, dO tiles; Q^T, dO^T images; 2 x 64 floats
 
+// Pre-pass: the accumulator start values of every 64-query tile, 128 floats per (batch, head, tile):
+// position 32*mt + 16*g + r holds -lse/scale of query acc_tile_row(r, g, mt) of the tile (-inf for
+// rows that must give P = 0: beyond Lq, or a query that saw no key), position 64 + ... its -delta.
+__global__ __launch_bounds__(128) void attn_bwd_stats_kernel(const AttnParams p, float* __restrict__ stats) {
+  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z, j = threadIdx.x & 63;
+  const int qi = t * KV_BQ + acc_tile_row(j & 15, (j >> 4) & 1, j >> 5);
+  const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
+  float v;
+  if (threadIdx.x < 64) {
+    float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
+    if (l == -INFINITY) l = INFINITY;
+    v = -l / p.scale;
+  } else {
+    v = (qi < p.Lq) ? -p.delta[ri] : 0.f;
+  }
+  stats[(((int64_t)b * p.Hq + h) * gridDim.x + t) * 128 + threadIdx.x] = v;
+}
+
 __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
                                                                          const bf16* __restrict__ qimg,
-                                                                         const bf16* __restrict__ doimg) {
+                                                                         const bf16* __restrict__ doimg,
+                                                                         const float* __restrict__ stats) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][KV_STAGE]
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
+            i = lane & 31;
   const BlockCoord bc = ody_block_coord(p.Hkv, p.B);   // rank 0 = first key block = most query tiles
   const int hk = bc.h, b = bc.b;
   const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
@@ -256,60 +276,39 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   const int t_begin = p.causal ? max(0, n0 - p.off) / KV_BQ : 0;   // first query tile that sees a key of this block
   const int ntq = max(0, q_tiles - t_begin);
   const int total = ntq * p.group;   // flattened (head of the group, query tile)
-  const float c2 = p.scale_log2e, inv_scale = 1.0f / p.scale;
+  const float c2 = p.scale_log2e;
   const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
 
+  // Direct loads of one stage: uniform base pointers plus 32-bit per-lane offsets that are
+  // recomputed from the lane id every time (cheaper than keeping them in registers here).
   auto load_stage = [&](bf16* st, int it) {
     const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
-    const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
-    const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
-    const bf16* qi_ = qimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
-    const bf16* doi = doimg + (((int64_t)b * p.Hq + h) * q_tiles + t) * IMG_ELEMS;
+    const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h + (int64_t)t * KV_BQ * p.sq.l;
+    const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h + (int64_t)t * KV_BQ * p.sdo.l;
+    const int64_t tile_id = ((int64_t)b * p.Hq + h) * q_tiles + t;
+    const bf16* qi_ = qimg + tile_id * IMG_ELEMS;
+    const bf16* doi = doimg + tile_id * IMG_ELEMS;
+    const int rmax = p.Lq - 1 - t * KV_BQ;   // rows beyond the matrix re-read its last row
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    if (wave == KV_WAVES - 1 && ln < 32)
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(stats + tile_id * 128 + (unsigned)(ln * 4)),
+                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS), 16, 0, 0);
 #pragma unroll
     for (int j = 0; j < 16 / KV_WAVES; j++) {
       const int grp = KV_WAVES * j + wave;
-      int row = t * KV_BQ + 4 * grp + (lane & 3);
-      row = row < p.Lq ? row : p.Lq - 1;
-      const int col = 8 * (lane >> 2);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (int64_t)row * p.sq.l + col),
+      const int row = min(4 * grp + (ln & 3), rmax), col = 8 * (ln >> 2);
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (unsigned)(row * (int)p.sq.l + col)),
                                        (lds_void_ptr)(st + grp * GROUP_ELEMS), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(dop + (int64_t)row * p.sdo.l + col),
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(dop + (unsigned)(row * (int)p.sdo.l + col)),
                                        (lds_void_ptr)(st + TILE_ELEMS + grp * GROUP_ELEMS), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(qi_ + (grp * 64 + lane) * 8),
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(qi_ + (unsigned)((grp * 64 + ln) * 8)),
                                        (lds_void_ptr)(st + 2 * TILE_ELEMS + grp * 512), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(doi + (grp * 64 + lane) * 8),
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(doi + (unsigned)((grp * 64 + ln) * 8)),
                                        (lds_void_ptr)(st + 2 * TILE_ELEMS + IMG_ELEMS + grp * 512), 16, 0, 0);
     }
   };
-  // the accumulator start values of the 64 queries of a tile, in accumulator order:
-  // position 32*mt + 16*g + r  <->  query acc_tile_row(r, g, mt).  -lse/scale (-inf for rows that
-  // must give P = 0: beyond Lq, or a query that saw no key) and -delta.
-  float lreg = 0.f, dreg = 0.f;
-  auto load_stats = [&](int it) {
-    if (tid < 64) {
-      const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
-      const int mt = tid >> 5, gg = (tid >> 4) & 1, r = tid & 15;
-      const int qi = t * KV_BQ + acc_tile_row(r, gg, mt);
-      const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
-      float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
-      if (l == -INFINITY) l = INFINITY;
-      lreg = -l * inv_scale;
-      dreg = (qi < p.Lq) ? -p.delta[ri] : 0.f;
-    }
-  };
-  auto store_stats = [&](bf16* st) {
-    if (tid < 64) {
-      float* f = reinterpret_cast<float*>(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS);
-      f[tid] = lreg;
-      f[64 + tid] = dreg;
-    }
-  };
-
-  if (total > 0) {
-    load_stage(ring, 0);
-    load_stats(0);
-    store_stats(ring);
-  }
+  if (total > 0) load_stage(ring, 0);
 
   // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
   // work, 16 MFMAs for dV^T and dK^T
@@ -377,10 +376,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     __syncthreads();
     const int t = q_tiles - 1 - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
                                               // Q / dO tiles at the same time and share them through L2
-    if (it + 1 < total) {
-      load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1);
-      load_stats(it + 1);
-    }
+    if (it + 1 < total) load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1);
     const bf16* st = ring + (it & 1) * KV_STAGE;
     // every query of the tile is before every key of this wavefront: nothing to do
     const bool dead = p.causal && (t * KV_BQ + KV_BQ - 1 + p.off < wn0);
@@ -389,7 +385,6 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 #pragma unroll 1
       for (int mt = 0; mt < 2; mt++) sub_tile(st, t, mt, masked);
     }
-    if (it + 1 < total) store_stats(ring + ((it + 1) & 1) * KV_STAGE);
   }
 
   if (key < p.Lk) {
@@ -415,9 +410,10 @@ inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 }  // namespace
 
-// workspace after delta: the transposed images of K, Q and dO
+// workspace after delta: the transposed images of K, Q and dO, and the per-tile start values
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
-  return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq));
+  return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq)) +
+         align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * 128 * sizeof(float));
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
@@ -439,12 +435,17 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   bf16* qimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)));
   bf16* doimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)) +
                                         align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
+  float* stats = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(doimg) +
+                                          align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
   int rc;
+  ODY_LAUNCH("attn_bwd_stats", st, attn_bwd_stats_kernel, dim3((p.Lq + KV_BQ - 1) / KV_BQ, p.Hq, p.B), dim3(128), 0, p,
+             stats);
+  if ((rc = ody_check_launch("attn_bwd_stats"))) return rc;
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
   if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
   if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
   dim3 gk(((p.Lk + KV_BN - 1) / KV_BN) * p.Hkv * p.B);
-  ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel, gk, dim3(KV_THREADS), smem_kv, p, qimg, doimg);
+  ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel, gk, dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats);
   if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
