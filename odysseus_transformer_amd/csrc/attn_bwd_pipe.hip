@@ -23,6 +23,30 @@ using namespace tile128;
 constexpr int D = 128, KS = D / 16, DT = D / 32;
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// The lane id, recomputed on the spot.  Where every register is spoken for, values derived from
+// it are cheaper to rebuild than to keep (the alternative is a spill to scratch memory, whose
+// reload then waits behind the tile loads in flight).
+__device__ __forceinline__ int fresh_lane() {
+  int ln;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+  return ln;
+}
+
+// Two wavefronts of a workgroup share each SIMD.  Started together and re-aligned by every
+// workgroup barrier they run in lockstep -- both in their matrix phase, then both in their
+// vector phase -- and the matrix pipe idles half of the time.  Raising the priority of the
+// first wavefront to arrive on each SIMD breaks the symmetry: it runs ahead, and the other
+// one fills the matrix pipe while the first is in its vector phase.
+__device__ __forceinline__ void simd_stagger(int tid) {
+  __shared__ int simd_count[4];
+  if (tid < 4) simd_count[tid] = 0;
+  __syncthreads();
+  const int simd = __builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4) & 3;   // HW_ID.SIMD_ID
+  int rank = 0;
+  if ((tid & 63) == 0) rank = atomicAdd(&simd_count[simd], 1);
+  if (__builtin_amdgcn_readfirstlane(rank) == 0) __builtin_amdgcn_s_setprio(2);
+}
+
 // ---------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------
@@ -214,34 +238,43 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 // ring as row tiles (A operands of S and dP) and as transposed images (A operands of dV^T and
 // dK^T); P and dS are accumulator tiles, which is the B-operand layout of the next product.
 //
-//      S  = Q K^T - lse/scale     the accumulator starts at -lse/scale, so P = exp2(S c)
-//      dP = dO V^T - delta        the accumulator starts at -delta
+//      S  = Q K^T - lse/scale     -lse/scale enters as one more k-step of the contraction, so P = exp2(S c)
+//      dP = dO V^T - delta        likewise -delta
 //      dV^T += dO^T P             dK^T += Q^T (P o dP)
 constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 * KV_WAVES;
-constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + 2 * 64 * 2;   // Q, dO tiles; Q^T, dO^T images; 2 x 64 floats
+constexpr int KV_STAT_ELEMS = 128 * 8;                                   // start-value fragments of one tile
+constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q, dO tiles; Q^T, dO^T images; start values
 
-// Pre-pass: the accumulator start values of every 64-query tile, 128 floats per (batch, head, tile):
-// position 32*mt + 16*g + r holds -lse/scale of query acc_tile_row(r, g, mt) of the tile (-inf for
-// rows that must give P = 0: beyond Lq, or a query that saw no key), position 64 + ... its -delta.
-__global__ __launch_bounds__(128) void attn_bwd_stats_kernel(const AttnParams p, float* __restrict__ stats) {
-  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z, j = threadIdx.x & 63;
-  const int qi = t * KV_BQ + acc_tile_row(j & 15, (j >> 4) & 1, j >> 5);
+// Pre-pass: the start values of S and dP for every 64-query tile, as one more A-operand
+// fragment of the contraction (the matching B fragment is all ones): the fp32 value x is split
+// into three bf16 terms x = h + m + l, which the MFMA adds up exactly like any other product.
+// Layout per (batch, head, tile): [sub-tile mt][0: -lse/scale, 1: -delta][MFMA row i][8 bf16],
+// row i of sub-tile mt being query tile_row(i, mt).  Rows that must give P = 0 (beyond Lq, or a
+// query that saw no key) get -1e30.
+__global__ __launch_bounds__(128) void attn_bwd_stats_kernel(const AttnParams p, bf16* __restrict__ stats) {
+  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int mt = threadIdx.x >> 6, which = (threadIdx.x >> 5) & 1, i = threadIdx.x & 31;
+  const int qi = t * KV_BQ + tile_row(i, mt);
   const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
-  float v;
-  if (threadIdx.x < 64) {
-    float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
-    if (l == -INFINITY) l = INFINITY;
-    v = -l / p.scale;
+  float x;
+  if (which == 0) {
+    const float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
+    x = (l == INFINITY || l == -INFINITY) ? -1e30f : -l / p.scale;
   } else {
-    v = (qi < p.Lq) ? -p.delta[ri] : 0.f;
+    x = (qi < p.Lq) ? -p.delta[ri] : 0.f;
   }
-  stats[(((int64_t)b * p.Hq + h) * gridDim.x + t) * 128 + threadIdx.x] = v;
+  const bf16 hi = (bf16)x;
+  const bf16 mid = (bf16)(x - (float)hi);
+  const bf16 lo = (bf16)(x - (float)hi - (float)mid);
+  const bf16 z = (bf16)0.f;
+  *reinterpret_cast<bf16x8*>(stats + ((((int64_t)b * p.Hq + h) * gridDim.x + t) * 128 + threadIdx.x) * 8) =
+      bf16x8{hi, mid, lo, z, z, z, z, z};
 }
 
 __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
                                                                          const bf16* __restrict__ qimg,
                                                                          const bf16* __restrict__ doimg,
-                                                                         const float* __restrict__ stats) {
+                                                                         const bf16* __restrict__ stats) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][KV_STAGE]
 
@@ -251,6 +284,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   const int hk = bc.h, b = bc.b;
   const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
   const int q_tiles = (p.Lq + KV_BQ - 1) / KV_BQ;
+  simd_stagger(tid);
 
   bf16x8 kf[KS], vf[KS];
   {
@@ -277,7 +311,6 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   const int ntq = max(0, q_tiles - t_begin);
   const int total = ntq * p.group;   // flattened (head of the group, query tile)
   const float c2 = p.scale_log2e;
-  const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
 
   // Direct loads of one stage: uniform base pointers plus 32-bit per-lane offsets that are
   // recomputed from the lane id every time (cheaper than keeping them in registers here).
@@ -289,11 +322,11 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     const bf16* qi_ = qimg + tile_id * IMG_ELEMS;
     const bf16* doi = doimg + tile_id * IMG_ELEMS;
     const int rmax = p.Lq - 1 - t * KV_BQ;   // rows beyond the matrix re-read its last row
-    int ln = lane;
-    asm volatile("" : "+v"(ln));
-    if (wave == KV_WAVES - 1 && ln < 32)
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(stats + tile_id * 128 + (unsigned)(ln * 4)),
-                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS), 16, 0, 0);
+    const int ln = fresh_lane();
+    if (wave >= KV_WAVES - 2)
+      __builtin_amdgcn_global_load_lds(
+          (global_void_ptr)(stats + tile_id * KV_STAT_ELEMS + (unsigned)(((wave - (KV_WAVES - 2)) * 64 + ln) * 8)),
+          (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS + (wave - (KV_WAVES - 2)) * 512), 16, 0, 0);
 #pragma unroll
     for (int j = 0; j < 16 / KV_WAVES; j++) {
       const int grp = KV_WAVES * j + wave;
@@ -313,20 +346,25 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
   // work, 16 MFMAs for dV^T and dK^T
   auto sub_tile = [&](const bf16* st, int t, int mt, bool masked) {
+    const int ln = fresh_lane(), g = ln >> 5, i = ln & 31;
+    const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
     const bf16* Qt = st;
     const bf16* Ot = st + TILE_ELEMS;
     const bf16* Qi = st + 2 * TILE_ELEMS;
     const bf16* Oi = Qi + IMG_ELEMS;
-    const float* Ls = reinterpret_cast<const float*>(Oi + IMG_ELEMS) + 32 * mt + 16 * g;
+    const bf16* St = Oi + IMG_ELEMS + mt * 512 + i * 8;
     constexpr int PF = 2;
     bf16x8 qfr[PF], ofr[PF];
-#pragma unroll
-    for (int n = 0; n < PF; n++) {
-      qfr[n] = row_frag(Qt, rbase, n, mt);
-      ofr[n] = row_frag(Ot, rbase, n, mt);
-    }
-    f32x16 s = *reinterpret_cast<const f32x16*>(Ls);
-    f32x16 dp = *reinterpret_cast<const f32x16*>(Ls + 64);
+    const bf16x8 s0 = *reinterpret_cast<const bf16x8*>(St), d0 = *reinterpret_cast<const bf16x8*>(St + 256);
+    qfr[0] = row_frag(Qt, rbase, 0, mt);
+    ofr[0] = row_frag(Ot, rbase, 0, mt);
+    const bf16 one = (bf16)(g == 0 ? 1.f : 0.f), zero = (bf16)0.f;
+    const bf16x8 ones = {one, one, one, zero, zero, zero, zero, zero};   // k-slots 0..2 carry the start value
+    FENCE();
+    f32x16 s = mfma32(s0, ones, f32x16{0});
+    f32x16 dp = mfma32(d0, ones, f32x16{0});
+    qfr[1] = row_frag(Qt, rbase, 1, mt);
+    ofr[1] = row_frag(Ot, rbase, 1, mt);
     FENCE();
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
@@ -345,7 +383,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
       qif[n] = image_frag(Qi, ibase, n & 3, n >> 2, mt);
     }
     if (masked) {
-      const int lim = key - p.off - t * KV_BQ;   // tile rows below lim come before this key
+      const int lim = wn0 + i - p.off - t * KV_BQ;   // tile rows below lim come before this lane's key
 #pragma unroll
       for (int r = 0; r < 16; r++)
         if (acc_tile_row(r, g, mt) < lim) s[r] = -INFINITY;
@@ -413,7 +451,7 @@ inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 // workspace after delta: the transposed images of K, Q and dO, and the per-tile start values
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
   return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq)) +
-         align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * 128 * sizeof(float));
+         align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16));
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
@@ -435,8 +473,8 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   bf16* qimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)));
   bf16* doimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)) +
                                         align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
-  float* stats = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(doimg) +
-                                          align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
+  bf16* stats = reinterpret_cast<bf16*>(reinterpret_cast<unsigned char*>(doimg) +
+                                        align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
   int rc;
   ODY_LAUNCH("attn_bwd_stats", st, attn_bwd_stats_kernel, dim3((p.Lq + KV_BQ - 1) / KV_BQ, p.Hq, p.B), dim3(128), 0, p,
              stats);
