@@ -51,6 +51,7 @@ __device__ __forceinline__ void simd_stagger(int tid) {
 // dQ
 // ---------------------------------------------------------------------------------
 constexpr int DQ_QT = 1, DQ_WAVES = 8, DQ_BM = 32 * DQ_QT * DQ_WAVES, DQ_THREADS = 64 * DQ_WAVES;
+static_assert(DQ_WAVES == 8, "the load split and the vmcnt waits assume 8 wavefronts");
 
 __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const AttnParams p,
                                                                        const bf16* __restrict__ kimg) {
@@ -59,7 +60,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* ring = reinterpret_cast<bf16*>(smem_raw);     // [3][STAGE]
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
+            i = lane & 31;
+  simd_stagger(tid);
   const BlockCoord bc = ody_block_coord(p.Hq, p.B);
   const int nqb = gridDim.x / (p.Hq * p.B);
   const int qblk = p.causal ? (nqb - 1 - bc.rank) : bc.rank;   // heaviest blocks first
@@ -81,9 +84,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   if (p.causal) n_full = min(n_full, max(0, (q0 + p.off + 1) / BN));
   n_full = min(n_full, ntiles);
 
-  auto load_stage = [&](bf16* st, int t) {
-#pragma unroll
-    for (int j = 0; j < 16 / DQ_WAVES; j++) {
+  auto load_part = [&](bf16* st, int t, int j) {   // j = 0, 1: the two halves of a stage's loads
+    {
       const int grp = DQ_WAVES * j + wave;
       int row = t * BN + 4 * grp + (lane & 3);
       row = row < p.Lk ? row : p.Lk - 1;
@@ -95,6 +97,10 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
       __builtin_amdgcn_global_load_lds((global_void_ptr)(kip + (int64_t)t * IMG_ELEMS + (grp * 64 + lane) * 8),
                                        (lds_void_ptr)(st + 2 * TILE_ELEMS + grp * 512), 16, 0, 0);
     }
+  };
+  auto load_stage = [&](bf16* st, int t) {
+    load_part(st, t, 0);
+    load_part(st, t, 1);
   };
   if (ntiles > 0) load_stage(ring, 0);
   if (ntiles > 1) load_stage(ring + STAGE, 1);
@@ -198,16 +204,17 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   for (int t = 0; t < ntiles; t++) {
     // stage t landed (the loads of stage t+1 may still be in flight), everyone done with stage t-1
     if (t + 1 < ntiles) {
-      if (DQ_WAVES == 8) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    }
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (t + 2 < ntiles) load_stage(ring + ((t + 2) % 3) * STAGE, t + 2);
     const bf16* st = ring + (t % 3) * STAGE;
-    if (p.causal && t * BN > wq0 + 32 * QT - 1 + p.off) continue;   // every key of the tile is after this wavefront's queries
+    const bool dead = p.causal && t * BN > wq0 + 32 * QT - 1 + p.off;   // every key of the tile is after this wavefront's queries
 #pragma unroll 1
-    for (int kt = 0; kt < 2; kt++) sub_tile(st, t, kt, t >= n_full);
+    for (int kt = 0; kt < 2; kt++) {
+      // half of the loads of stage t+2 before each sub-tile (all at once they queue up at the memory pipeline)
+      if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, kt);
+      if (!dead) sub_tile(st, t, kt, t >= n_full);
+    }
   }
 
 #pragma unroll
@@ -314,7 +321,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 
   // Direct loads of one stage: uniform base pointers plus 32-bit per-lane offsets that are
   // recomputed from the lane id every time (cheaper than keeping them in registers here).
-  auto load_stage = [&](bf16* st, int it) {
+  auto load_stage = [&](bf16* st, int it, int j) {   // j = 0, 1: the two halves of the stage's loads
     const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
     const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h + (int64_t)t * KV_BQ * p.sq.l;
     const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h + (int64_t)t * KV_BQ * p.sdo.l;
@@ -323,12 +330,11 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     const bf16* doi = doimg + tile_id * IMG_ELEMS;
     const int rmax = p.Lq - 1 - t * KV_BQ;   // rows beyond the matrix re-read its last row
     const int ln = fresh_lane();
-    if (wave >= KV_WAVES - 2)
+    if (j == 0 && wave >= KV_WAVES - 2)
       __builtin_amdgcn_global_load_lds(
           (global_void_ptr)(stats + tile_id * KV_STAT_ELEMS + (unsigned)(((wave - (KV_WAVES - 2)) * 64 + ln) * 8)),
           (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS + (wave - (KV_WAVES - 2)) * 512), 16, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 16 / KV_WAVES; j++) {
+    {
       const int grp = KV_WAVES * j + wave;
       const int row = min(4 * grp + (ln & 3), rmax), col = 8 * (ln >> 2);
       __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (unsigned)(row * (int)p.sq.l + col)),
@@ -341,7 +347,10 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
                                        (lds_void_ptr)(st + 2 * TILE_ELEMS + IMG_ELEMS + grp * 512), 16, 0, 0);
     }
   };
-  if (total > 0) load_stage(ring, 0);
+  if (total > 0) {
+    load_stage(ring, 0, 0);
+    load_stage(ring, 0, 1);
+  }
 
   // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
   // work, 16 MFMAs for dV^T and dK^T
@@ -414,14 +423,16 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     __syncthreads();
     const int t = q_tiles - 1 - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
                                               // Q / dO tiles at the same time and share them through L2
-    if (it + 1 < total) load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1);
     const bf16* st = ring + (it & 1) * KV_STAGE;
     // every query of the tile is before every key of this wavefront: nothing to do
     const bool dead = p.causal && (t * KV_BQ + KV_BQ - 1 + p.off < wn0);
-    if (!dead) {
-      const bool masked = p.causal && (t * KV_BQ + p.off < wn0 + 31);
+    const bool masked = p.causal && (t * KV_BQ + p.off < wn0 + 31);
 #pragma unroll 1
-      for (int mt = 0; mt < 2; mt++) sub_tile(st, t, mt, masked);
+    for (int mt = 0; mt < 2; mt++) {
+      // the loads of the next stage go out in two halves, one before each sub-tile: issued all at
+      // once by eight wavefronts they would queue up behind each other at the memory pipeline
+      if (it + 1 < total) load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1, mt);
+      if (!dead) sub_tile(st, t, mt, masked);
     }
   }
 
