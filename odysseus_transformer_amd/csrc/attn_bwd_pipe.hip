@@ -87,9 +87,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   auto load_part = [&](bf16* st, int t, int j) {   // j = 0, 1: the two halves of a stage's loads
     {
       const int grp = DQ_WAVES * j + wave;
-      int row = t * BN + 4 * grp + (lane & 3);
+      int row = t * BN + 4 * grp + (lane >> 4);
       row = row < p.Lk ? row : p.Lk - 1;
-      const int col = 8 * (lane >> 2);
+      const int col = 8 * (lane & 15);
       __builtin_amdgcn_global_load_lds((global_void_ptr)(kp + (int64_t)row * p.sk.l + col),
                                        (lds_void_ptr)(st + grp * GROUP_ELEMS), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((global_void_ptr)(vp + (int64_t)row * p.sv.l + col),
@@ -142,8 +142,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   // one 32-key sub-tile x 64 queries: 32 MFMAs for S^T and dP^T, the vector work, 16 MFMAs for
   // dQ^T; every LDS operand fragment feeds two MFMAs
   auto sub_tile = [&](const bf16* st, int t, int kt, bool masked) {
-    const bf16* Kt = st + kt * 16;
-    const bf16* Vt = st + TILE_ELEMS + kt * 16;
+    const bf16* Kt = st + kt * KT_ELEMS;
+    const bf16* Vt = st + TILE_ELEMS + kt * KT_ELEMS;
     const bf16* Ki = st + 2 * TILE_ELEMS + kt * 512;
     constexpr int PF = 3;
     bf16x8 kfr[PF], vfr[PF];
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
           (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS + (wave - (KV_WAVES - 2)) * 512), 16, 0, 0);
     {
       const int grp = KV_WAVES * j + wave;
-      const int row = min(4 * grp + (ln & 3), rmax), col = 8 * (ln >> 2);
+      const int row = min(4 * grp + (ln >> 4), rmax), col = 8 * (ln & 15);
       __builtin_amdgcn_global_load_lds((global_void_ptr)(qp + (unsigned)(row * (int)p.sq.l + col)),
                                        (lds_void_ptr)(st + grp * GROUP_ELEMS), 16, 0, 0);
       __builtin_amdgcn_global_load_lds((global_void_ptr)(dop + (unsigned)(row * (int)p.sdo.l + col)),

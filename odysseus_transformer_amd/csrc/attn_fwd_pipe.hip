@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
   bf16* Kring = reinterpret_cast<bf16*>(smem_raw);   // [3][TILE_ELEMS]
   bf16* Vring = Kring + 3 * TILE_ELEMS;              // [2][IMG_ELEMS]
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 5, i = lane & 31;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5, i = lane & 31;
   const BlockCoord bc = ody_block_coord(p.Hq, p.B);
   const int nqb = gridDim.x / (p.Hq * p.B);
   const int qblk = p.causal ? (nqb - 1 - bc.rank) : bc.rank;   // heaviest blocks first
@@ -109,10 +109,10 @@ __global__ __launch_bounds__(256) void attn_fwd_pipe_kernel(const AttnParams p, 
 
   f32x16 sA[QT], sB[QT];
 
-  // per-thread element offsets of the 4 direct loads of a K tile (rows 4*grp + (lane & 3), chunk lane >> 2)
+  // per-thread element offsets of the 4 direct loads of a K tile (row 4*grp + (lane >> 4), chunk lane & 15)
   unsigned koff[4];
 #pragma unroll
-  for (int j = 0; j < 4; j++) koff[j] = (unsigned)((4 * (4 * j + wave) + (lane & 3)) * p.sk.l + 8 * (lane >> 2));
+  for (int j = 0; j < 4; j++) koff[j] = (unsigned)((4 * (4 * j + wave) + (lane >> 4)) * p.sk.l + 8 * (lane & 15));
   // a K tile whose 64 rows all exist: uniform base + per-lane offset; the ragged last tile clamps rows
   auto load_k = [&](bf16* lds_tile, int row0) {
     if (row0 + ROWS <= p.Lk) {

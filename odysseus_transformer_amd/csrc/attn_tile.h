@@ -4,17 +4,21 @@
 //
 // A direct load (global_load_lds_dwordx4) makes the 64 lanes of a wavefront write
 // 64 consecutive 16-byte slots of LDS, each lane fetching from its own global
-// address.  One such load brings a GROUP of 4 consecutive tile rows (4 x 256 B);
-// inside the group the slots are chunk-major: slot = chunk * 4 + (row & 3), where a
-// chunk is 8 consecutive bf16 of a row.  Groups are 1040 bytes apart (1024 + 16 of
-// padding).  Hence, in elements,
+// address.  One such load brings a GROUP of 4 consecutive tile rows (4 x 256 B), row
+// after row; groups are 1040 bytes apart (1024 + 16 of padding).  Hence, in elements,
 //
-//     offset(row, col) = (row >> 2) * 520 + (col >> 3) * 32 + (row & 3) * 8 + (col & 7)
+//     offset(row, col) = (row >> 2) * 520 + (row & 3) * 128 + col
 //
-// The 16 lanes that are served together read the same chunk of rows 4*i + b
-// (i = 0..15, b fixed): their addresses are 1040 bytes apart, i.e. 4 banks apart ->
-// 64 distinct banks.  For that, row rho (0..31) of a 32-row MFMA operand of sub-tile
-// kt (0/1) is tile row  4*(rho & 15) + (rho >> 4) + 2*kt.
+// How the LDS serves a 16-byte read (measured on gfx950): the two halves of the wavefront
+// go separately; within a half of 32 lanes, lanes whose index has an even number of ones in
+// bits 2, 3 and 4 (lanes 0-3, 12-15, 20-27) are served together, and so are the other 16.
+// Each such set must touch every one of the 64 banks once (a lane covers 4 consecutive
+// banks).  A pattern where lane i + 16 is a multiple of 256 bytes away from lane i, and lanes
+// 0..15 cover 16 different 16-byte slots modulo 256 bytes, satisfies that.  Here lanes 0..15
+// read the same chunk of rows 4*i + b (b fixed): 1040 bytes apart, i.e. one slot apart modulo
+// 256; lanes 16..31 read row 4*i + b + 1, exactly 256 bytes further.  For that, row rho
+// (0..31) of a 32-row MFMA operand of sub-tile kt (0/1) is tile row
+// 4*(rho & 15) + (rho >> 4) + 2*kt.
 #pragma once
 #include "ody_common.h"
 
@@ -45,19 +49,20 @@ __device__ __forceinline__ void load_tile_async(bf16* lds_tile, const bf16* base
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     const int grp = 4 * j + wave;
-    int row = row0 + 4 * grp + (lane & 3);
+    int row = row0 + 4 * grp + (lane >> 4);
     row = row < nrows ? row : nrows - 1;
-    const bf16* src = base + (int64_t)row * row_stride + 8 * (lane >> 2);
+    const bf16* src = base + (int64_t)row * row_stride + 8 * (lane & 15);
     __builtin_amdgcn_global_load_lds((global_void_ptr)src, (lds_void_ptr)(lds_tile + grp * GROUP_ELEMS), 16, 0, 0);
   }
 }
 
 // Per-lane element offset of the row-wise operand: MFMA row i, k = 8g..8g+7 of k-step 0,
-// sub-tile 0.  Add ks*64 + kt*16 elements for k-step ks of sub-tile kt.
-__device__ __forceinline__ int row_frag_base(int g, int i) { return (i & 15) * GROUP_ELEMS + g * 32 + (i >> 4) * 8; }
+// sub-tile 0.  Add ks*16 + kt*KT_ELEMS elements for k-step ks of sub-tile kt.
+constexpr int KT_ELEMS = 256;                    // sub-tile 1 starts two rows further
+__device__ __forceinline__ int row_frag_base(int g, int i) { return (i & 15) * GROUP_ELEMS + (i >> 4) * 128 + g * 8; }
 
 __device__ __forceinline__ bf16x8 row_frag(const bf16* tile, int base, int ks, int kt) {
-  return *reinterpret_cast<const bf16x8*>(tile + base + ks * 64 + kt * 16);
+  return *reinterpret_cast<const bf16x8*>(tile + base + ks * 16 + kt * KT_ELEMS);
 }
 
 // ---------------------------------------------------------------------------------
