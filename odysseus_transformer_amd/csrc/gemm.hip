@@ -13,6 +13,7 @@
 //
 // fp32: 64 x 64 tiles on the vector ALUs (the fp32 configuration is small and
 // its 1e-4 tolerance rules out bf16 inputs).
+#include <type_traits>
 #include "ody_common.h"
 
 namespace {
@@ -64,6 +65,176 @@ struct OperandTile {
     }
   }
 };
+
+// Interior tiles with K a multiple of 64 take this kernel.  Same tiles and fragments as the
+// general kernel below, but the traffic of the next slabs is spread over the MFMA stream
+// instead of being issued in bursts: a wavefront is held up while the memory pipeline accepts
+// its loads (64 bytes per clock per CU) and while the LDS takes its writes, and with one
+// wavefront per SIMD the matrix pipe idles meanwhile.  Per 16-MFMA k-step the wavefront issues
+// a quarter of the global loads of slab kt+2 (into one of two register sets), a quarter of the
+// LDS writes of slab kt+1 (from the other set, loaded one iteration earlier) and the fragment
+// reads of the next k-step.
+#define GEMM_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+template <int WM, int WN, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
+                                                             bf16* __restrict__ C, const bf16* __restrict__ bias,
+                                                             int M, int N, int K, int64_t lda, int64_t ldb,
+                                                             int64_t ldc, int accumulate, int tiles_m, int tiles_n) {
+  constexpr int TM = 64 * WM, TN = 64 * WN;
+  typedef OperandTile<TM, A_KC> TA;
+  typedef OperandTile<TN, B_KC> TB;
+  constexpr int CA = TA::CHUNKS, CB = TB::CHUNKS, KSTEPS = BK / 16;
+  static_assert(CA % KSTEPS == 0 && CB % KSTEPS == 0, "chunks are issued a quarter per k-step");
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* As = reinterpret_cast<bf16*>(smem_raw);  // [2][TA::ELEMS]
+  bf16* Bs = As + 2 * TA::ELEMS;                 // [2][TB::ELEMS]
+
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
+            i = lane & 31;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  int pid = blockIdx.x;
+  const int nblk = tiles_m * tiles_n;
+  if (nblk % 8 == 0) pid = (pid % 8) * (nblk / 8) + pid / 8;
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int gid = pid / per_group, first_m = gid * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int tm = first_m + (pid % per_group) % gsz, tn = (pid % per_group) / gsz;
+  const int m0 = tm * TM, n0 = tn * TN;
+
+  // chunk j of a thread: global element offset = off0 + j * step (+ slab advance), LDS element offset = lds0 + j * lstep
+  unsigned a_off0, b_off0, a_lds0, b_lds0;
+  int64_t a_step, b_step, a_slab, b_slab;
+  int a_lstep, b_lstep;
+  if (A_KC) {
+    a_off0 = (unsigned)((tid / 8) * lda + (tid % 8) * 8); a_step = 32 * lda; a_slab = BK;
+    a_lds0 = (tid / 8) * TA::PITCH + (tid % 8) * 8; a_lstep = 32 * TA::PITCH;
+  } else {
+    a_off0 = (unsigned)((tid / (TM / 8)) * lda + (tid % (TM / 8)) * 8); a_step = (256 / (TM / 8)) * lda; a_slab = BK * lda;
+    a_lds0 = (tid / (TM / 8)) * TA::PITCH + (tid % (TM / 8)) * 8; a_lstep = (256 / (TM / 8)) * TA::PITCH;
+  }
+  if (B_KC) {
+    b_off0 = (unsigned)((tid / 8) * ldb + (tid % 8) * 8); b_step = 32 * ldb; b_slab = BK;
+    b_lds0 = (tid / 8) * TB::PITCH + (tid % 8) * 8; b_lstep = 32 * TB::PITCH;
+  } else {
+    b_off0 = (unsigned)((tid / (TN / 8)) * ldb + (tid % (TN / 8)) * 8); b_step = (256 / (TN / 8)) * ldb; b_slab = BK * ldb;
+    b_lds0 = (tid / (TN / 8)) * TB::PITCH + (tid % (TN / 8)) * 8; b_lstep = (256 / (TN / 8)) * TB::PITCH;
+  }
+  const bf16* Abase = A_KC ? A + (int64_t)m0 * lda : A + m0;   // first element of the tile's slab 0
+  const bf16* Bbase = B_KC ? B + (int64_t)n0 * ldb : B + n0;
+
+  f32x16 acc[WM][WN];
+#pragma unroll
+  for (int a = 0; a < WM; a++)
+#pragma unroll
+    for (int b = 0; b < WN; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+
+  bf16x8 ra[CA], rb[CB];
+  auto gload_a = [&](int kt, int j) {
+    ra[j] = *reinterpret_cast<const bf16x8*>(Abase + (int64_t)kt * a_slab + j * a_step + a_off0);
+  };
+  auto gload_b = [&](int kt, int j) {
+    rb[j] = *reinterpret_cast<const bf16x8*>(Bbase + (int64_t)kt * b_slab + j * b_step + b_off0);
+  };
+  auto sstore_a = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(As + buf * TA::ELEMS + a_lds0 + j * a_lstep) = ra[j]; };
+  auto sstore_b = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(Bs + buf * TB::ELEMS + b_lds0 + j * b_lstep) = rb[j]; };
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int j = 0; j < CA; j++) gload_a(0, j);
+#pragma unroll
+  for (int j = 0; j < CB; j++) gload_b(0, j);
+#pragma unroll
+  for (int j = 0; j < CA; j++) sstore_a(0, j);
+#pragma unroll
+  for (int j = 0; j < CB; j++) sstore_b(0, j);
+  {
+    const int k1 = min(1, nk - 1);
+#pragma unroll
+    for (int j = 0; j < CA; j++) gload_a(k1, j);
+#pragma unroll
+    for (int j = 0; j < CB; j++) gload_b(k1, j);
+  }
+  __syncthreads();
+
+  // Slab kt is in LDS buffer kt & 1 and the registers hold slab kt+1.  Per k-step a quarter of
+  // the registers goes to the other LDS buffer and is refilled at once with its part of slab kt+2.
+  for (int kt = 0; kt < nk; kt++) {
+    const int buf = kt & 1;
+    const bf16* Ab = As + buf * TA::ELEMS;
+    const bf16* Bb = Bs + buf * TB::ELEMS;
+    const int kt2 = min(kt + 2, nk - 1);   // past the end: a harmless re-load, and a write nobody reads
+    bf16x8 af[2][WM], bfr[2][WN];
+#pragma unroll
+    for (int a = 0; a < WM; a++) af[0][a] = TA::frag(Ab, 32 * (wm * WM + a), 0, g, i);
+#pragma unroll
+    for (int b = 0; b < WN; b++) bfr[0][b] = TB::frag(Bb, 32 * (wn * WN + b), 0, g, i);
+    GEMM_FENCE();
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+#pragma unroll
+      for (int a = 0; a < WM; a++) {
+#pragma unroll
+        for (int b = 0; b < WN; b++) acc[a][b] = mfma32(bfr[cur][b], af[cur][a], acc[a][b]);  // rows = n, cols = m
+        if (ks + 1 < KSTEPS) {
+          af[nxt][a] = TA::frag(Ab, 32 * (wm * WM + a), ks + 1, g, i);
+          if (a < WN) bfr[nxt][a] = TB::frag(Bb, 32 * (wn * WN + a), ks + 1, g, i);
+        }
+        // chunks [ks * C / KSTEPS, (ks + 1) * C / KSTEPS) of both operands, spread over the WM groups of MFMAs
+#pragma unroll
+        for (int j = ks * (CA / KSTEPS); j < (ks + 1) * (CA / KSTEPS); j++)
+          if ((j - ks * (CA / KSTEPS)) * WM / (CA / KSTEPS) == a) {
+            sstore_a(buf ^ 1, j);
+            gload_a(kt2, j);
+          }
+#pragma unroll
+        for (int j = ks * (CB / KSTEPS); j < (ks + 1) * (CB / KSTEPS); j++)
+          if ((j - ks * (CB / KSTEPS)) * WM / (CB / KSTEPS) == a) {
+            sstore_b(buf ^ 1, j);
+            gload_b(kt2, j);
+          }
+        GEMM_FENCE();
+      }
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane (g, i) holds column m = i, rows n = 8*(r/4) + 4g + r%4
+#pragma unroll
+  for (int a = 0; a < WM; a++) {
+    const int m = m0 + 32 * (wm * WM + a) + i;
+#pragma unroll
+    for (int b = 0; b < WN; b++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + 32 * (wn * WN + b) + 8 * q + 4 * g;
+        bf16* dst = C + (int64_t)m * ldc + n;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+        if (bias) {
+          const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n);
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+        }
+        if (accumulate) {
+          const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)old[e];
+        }
+        bf16x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = (bf16)v[e];
+        *reinterpret_cast<bf16x4*>(dst) = w;
+      }
+    }
+  }
+}
 
 template <int WM, int WN, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
@@ -178,9 +349,13 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
   constexpr size_t smem = 2 * sizeof(bf16) * (OperandTile<TM, A_KC>::ELEMS + OperandTile<TN, B_KC>::ELEMS);
   static bool attr_set = false;
   auto kern = &gemm_bf16_kernel<WM, WN, A_KC, B_KC>;
+  auto fast = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC>;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)smem);
     if (e != hipSuccess) {
       ody_set_error("ody_gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
       return ODY_ERR_LAUNCH;
@@ -189,6 +364,15 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
   }
   const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
   const char* name = A_KC ? (B_KC ? "gemm_bf16_nt" : "gemm_bf16_nn") : "gemm_bf16_tn";
+  // per-thread offsets inside a tile are kept in 32 bits by the fast kernel
+  const bool interior = M % TM == 0 && N % TN == 0 && K % BK == 0 && (int64_t)TM * lda < (1ll << 31) &&
+                        (int64_t)TN * ldb < (1ll << 31) && (int64_t)BK * lda < (1ll << 31) &&
+                        (int64_t)BK * ldb < (1ll << 31);
+  if (interior) {
+    ODY_LAUNCH(name, st, fast, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
+               accumulate, tiles_m, tiles_n);
+    return ody_check_launch("gemm_bf16");
+  }
   ODY_LAUNCH(name, st, kern, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
              accumulate, tiles_m, tiles_n);
   return ody_check_launch("gemm_bf16");
