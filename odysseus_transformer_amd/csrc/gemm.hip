@@ -204,7 +204,45 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     __syncthreads();
   }
 
-  // epilogue: lane (g, i) holds column m = i, rows n = 8*(r/4) + 4g + r%4
+  // Epilogue.  Lane (g, i) holds column m = i and rows n = 8*(r/4) + 4g + r%4 of each 32 x 32 tile,
+  // i.e. 8-byte pieces of 32 different rows of C.  Unless C is accumulated into, the tiles go
+  // through LDS (free by now) one 32-row band at a time and leave as 16-byte pieces of whole rows.
+  if (!accumulate) {
+    constexpr int EP = 32 * WN + 8;                                     // band pitch in elements
+    bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;   // 32 rows x (32 * WN) columns per wavefront
+    static_assert(4 * 32 * EP <= 2 * (TA::ELEMS + TB::ELEMS), "the bands fit in the operand buffers");
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int nl = 32 * b + 8 * q + 4 * g;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          if (bias) {
+            const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n0 + 32 * wn * WN + nl);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+          }
+          bf16x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; e++) w[e] = (bf16)v[e];
+          *reinterpret_cast<bf16x4*>(band + i * EP + nl) = w;
+        }
+      // the band is private to the wavefront and LDS operations of a wavefront complete in order
+      constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;                  // 16-byte chunks per row, rows per pass
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const bf16x8 w = *reinterpret_cast<const bf16x8*>(band + row * EP + 8 * c);
+        const int m = m0 + 32 * (wm * WM + a) + row;
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + n0 + 32 * wn * WN + 8 * c) = w;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < WM; a++) {
     const int m = m0 + 32 * (wm * WM + a) + i;
@@ -364,8 +402,9 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
   }
   const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
   const char* name = A_KC ? (B_KC ? "gemm_bf16_nt" : "gemm_bf16_nn") : "gemm_bf16_tn";
-  // per-thread offsets inside a tile are kept in 32 bits by the fast kernel
+  // per-thread offsets inside a tile are kept in 32 bits by the fast kernel, and it writes C in 16-byte pieces
   const bool interior = M % TM == 0 && N % TN == 0 && K % BK == 0 && (int64_t)TM * lda < (1ll << 31) &&
+                        ody_aligned16(C) && ldc % 8 == 0 &&
                         (int64_t)TN * ldb < (1ll << 31) && (int64_t)BK * lda < (1ll << 31) &&
                         (int64_t)BK * ldb < (1ll << 31);
   if (interior) {

@@ -11,6 +11,8 @@ SHAPES = [
     # M, N, K
     (64, 64, 64),
     (256, 256, 256),
+    (128, 128, 64),        # interior tiles, a single K slab
+    (256, 384, 192),       # interior tiles, odd number of K slabs
     (300, 136, 72),        # ragged in every direction (multiples of 8)
     (2048, 1536, 512),     # the fp32 configuration's QKV projection
     (520, 2752, 512),      # gate_up of the fp32 configuration, ragged M
@@ -55,6 +57,29 @@ def test_bias_accumulate_and_strides(dtype, dev):
     out = c0.to(dev).clone()
     ops.gemm(ops.GEMM_NT, xg, w.to(dev), bias=b.to(dev), out=out, accumulate=True)
     assert rel_err(out, ref) <= tol
+
+
+@pytest.mark.parametrize("op", ["nt", "nn", "tn"])
+def test_bias_accumulate_and_strides_on_interior_tiles(op, dev):
+    """The kernel for full tiles: padded leading dimensions, bias and accumulation into C."""
+    from odysseus_transformer_amd import ops
+    dt = torch.bfloat16
+    M, N, K = 512, 256, 320
+    shape_a = {"nt": (M, K), "nn": (M, K), "tn": (K, M)}[op]
+    shape_b = {"nt": (N, K), "nn": (K, N), "tn": (K, N)}[op]
+    a = randn((shape_a[0], shape_a[1] + 40), 11, dtype=dt)[:, 16:16 + shape_a[1]]
+    b = randn((shape_b[0], shape_b[1] + 8), 12, std=0.05, dtype=dt)[:, :shape_b[1]]
+    bias = randn((N,), 13, dtype=dt)
+    c0 = randn((M, N + 16), 14, dtype=dt)[:, 8:8 + N]
+    af = a.float().t() if op == "tn" else a.float()
+    bf = b.float().t() if op == "nt" else b.float()
+    ref = af @ bf + bias.float() + c0.float()
+    ag = randn((shape_a[0], shape_a[1] + 40), 11, dtype=dt).to(dev)[:, 16:16 + shape_a[1]]
+    bg = randn((shape_b[0], shape_b[1] + 8), 12, std=0.05, dtype=dt).to(dev)[:, :shape_b[1]]
+    out = randn((M, N + 16), 14, dtype=dt).to(dev)[:, 8:8 + N]
+    code = {"nt": ops.GEMM_NT, "nn": ops.GEMM_NN, "tn": ops.GEMM_TN}[op]
+    ops.gemm(code, ag, bg, bias=bias.to(dev), out=out, accumulate=True)
+    assert rel_err(out, ref) <= TOL_BF16
 
 
 def test_linearity_at_full_size(dev):
