@@ -158,14 +158,23 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
   }
 }
 
+// out[c] = sum_r partial[r][c].  A block owns 16 columns (64-byte row pieces) and splits the rows
+// over 16 thread groups, so that d / 16 blocks share the reading.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_kernel(const float* __restrict__ partial, T* __restrict__ out, int n,
                                                      int d) {
-  const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= d) return;
+  __shared__ float red[16][17];
+  const int cl = threadIdx.x & 15, rg = threadIdx.x >> 4, c = blockIdx.x * 16 + cl;
   float s = 0.f;
-  for (int r = 0; r < n; r++) s += partial[(int64_t)r * d + c];
-  out[c] = (T)s;
+  if (c < d)
+    for (int r = rg; r < n; r += 16) s += partial[(int64_t)r * d + c];
+  red[rg][cl] = s;
+  __syncthreads();
+  if (rg == 0 && c < d) {
+#pragma unroll
+    for (int k = 1; k < 16; k++) s += red[k][cl];
+    out[c] = (T)s;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -357,9 +366,9 @@ extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, 
   int rc = ody_check_launch("rmsnorm_bwd");
   if (rc || !dw) return rc;
   ODY_BY_DTYPE(dtype,
-               ODY_LAUNCH("colsum", st, colsum_kernel<bf16>, dim3((d + 255) / 256), dim3(256), 0, dw_partial, (bf16*)dw,
+               ODY_LAUNCH("colsum", st, colsum_kernel<bf16>, dim3((d + 15) / 16), dim3(256), 0, dw_partial, (bf16*)dw,
                                   nblocks, d),
-               ODY_LAUNCH("colsum", st, colsum_kernel<float>, dim3((d + 255) / 256), dim3(256), 0, dw_partial,
+               ODY_LAUNCH("colsum", st, colsum_kernel<float>, dim3((d + 15) / 16), dim3(256), 0, dw_partial,
                                   (float*)dw, nblocks, d));
   return ody_check_launch("rmsnorm_bwd_colsum");
 }
