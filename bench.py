@@ -168,7 +168,7 @@ def main():
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "causal attention fwd+bwd, Llama-2-7B rank shard at N=8: 4 heads x 128, L=32768, "
-                               "batch 1 (BASELINE.json configs[1], attention part)",
+                               "batch 1 (attention part of the 32768-token bf16 configuration)",
                    "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd},
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "device": {"name": prop.name, "cus": prop.multi_processor_count,

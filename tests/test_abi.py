@@ -53,3 +53,27 @@ def test_product_package_never_imports_the_oracle():
     pkg = ROOT / "odysseus_transformer_amd"
     for f in pkg.rglob("*.py"):
         assert "oracle" not in f.read_text(), f"{f} mentions the oracle"
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """No fallback: with the shared library absent every kernel call raises (checked in a fresh
+    interpreter so that the handle this process has already loaded plays no part)."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, torch\n"
+        f"sys.path.insert(0, {str(ROOT)!r})\n"
+        "from odysseus_transformer_amd import ops, _lib\n"
+        "try:\n"
+        "    _lib.load()\n"
+        "except ImportError as e:\n"
+        "    print('LOAD', type(e).__name__)\n"
+        "try:\n"
+        "    ops.gemm(ops.GEMM_NT, torch.zeros(8, 8), torch.zeros(8, 8))\n"
+        "except Exception as e:\n"
+        "    print('OP', type(e).__name__)\n"
+    )
+    env = dict(**__import__("os").environ, ODYSSEUS_HIP_LIB=str(tmp_path / "absent.so"))
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120).stdout
+    assert "LOAD ImportError" in out
+    assert "OP " in out and "OP None" not in out
