@@ -1,5 +1,6 @@
 // extern "C" entry points for attention.
 #include <cmath>
+#include <cstdlib>
 #include "attn_params.h"
 
 namespace {
@@ -62,7 +63,8 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
                 workspace_bytes, need);
     ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
                 "ody_attn_fwd: workspace must be 256-byte aligned");
-    return ody_launch_attn_fwd_pipe(p, workspace, st);
+    if (getenv("ODY_FWD_OLD")) return ody_launch_attn_fwd_pipe(p, workspace, st);
+    return ody_launch_attn_fwd_w8(p, workspace, st);
   }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
   return ody_launch_attn_fwd_simt(p, D, dtype, st);

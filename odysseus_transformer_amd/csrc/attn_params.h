@@ -51,6 +51,9 @@ size_t ody_attn_images_bytes(int B, int L, int H);
 int ody_launch_attn_images(const void* src, const AttnStrides& s, int B, int L, int H, void* dst, int* flags,
                            int nflags, hipStream_t st);
 size_t ody_attn_fwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
+// the same with 8 wavefronts x 32 queries per block; same workspace layout
+int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, hipStream_t st);
+size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
 // the online-rescaling forward kernel restricted to query blocks of `block` rows whose flag is set
 int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st);
 // head_dim 128 only; workspace of ody_attn_bwd_pipe_workspace(...) bytes (p.delta is set separately)

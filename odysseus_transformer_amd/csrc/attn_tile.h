@@ -112,6 +112,30 @@ __device__ __forceinline__ bf16x8 image_frag(const bf16* img, int base, int dt, 
 
 }  // namespace tile128
 
+// The lane id, recomputed on the spot.  Where every register is spoken for, values derived from
+// it are cheaper to rebuild than to keep (the alternative is a spill to scratch memory, whose
+// reload then waits behind the tile loads in flight).
+__device__ __forceinline__ int fresh_lane() {
+  int ln;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+  return ln;
+}
+
+// Two wavefronts of a workgroup share each SIMD.  Started together and re-aligned by every
+// workgroup barrier they run in lockstep -- both in their matrix phase, then both in their
+// vector phase -- and the matrix pipe idles half of the time.  Raising the priority of the
+// first wavefront to arrive on each SIMD breaks the symmetry: it runs ahead, and the other
+// one fills the matrix pipe while the first is in its vector phase.
+__device__ __forceinline__ void simd_stagger(int tid) {
+  __shared__ int simd_count[4];
+  if (tid < 4) simd_count[tid] = 0;
+  __syncthreads();
+  const int simd = __builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4) & 3;   // HW_ID.SIMD_ID
+  int rank = 0;
+  if ((tid & 63) == 0) rank = atomicAdd(&simd_count[simd], 1);
+  if (__builtin_amdgcn_readfirstlane(rank) == 0) __builtin_amdgcn_s_setprio(2);
+}
+
 // Swap of the two wavefront halves through v_permlane32_swap: returns, in every lane,
 // op(x of this lane, x of the lane 32 away).
 __device__ __forceinline__ float half_swap_max(float x) {
