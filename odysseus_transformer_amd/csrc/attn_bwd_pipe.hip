@@ -115,64 +115,72 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 #pragma unroll
       for (int r = 0; r < 16; r++) dq[qt][dt][r] = 0.f;
 
-  // one 32-key sub-tile x 64 queries: 32 MFMAs for S^T and dP^T, the vector work, 16 MFMAs for
-  // dQ^T; every LDS operand fragment feeds two MFMAs
-  auto sub_tile = [&](const bf16* st, int t, int kt, bool masked) {
-    const bf16* Kt = st + kt * KT_ELEMS;
-    const bf16* Vt = st + TILE_ELEMS + kt * KT_ELEMS;
-    const bf16* Ki = st + 2 * TILE_ELEMS + kt * 512;
-    constexpr int PF = 3;
-    bf16x8 kfr[PF], vfr[PF];
+  // One 64-key tile against this wavefront's 32 queries, as two 32-key sub-tiles kt = 0, 1 with their
+  // own accumulation chains: 32 MFMAs for S^T and dP^T, the vector work, 16 MFMAs for dQ^T.
+  auto tile = [&](const bf16* st, int t, bool masked) {
+    const bf16* Kt = st;
+    const bf16* Vt = st + TILE_ELEMS;
+    const bf16* Ki = st + 2 * TILE_ELEMS;
+    constexpr int PF = 2;
+    bf16x8 kfr[PF][2], vfr[PF][2];
 #pragma unroll
-    for (int n = 0; n < PF; n++) {
-      kfr[n] = row_frag(Kt, rbase, n, 0);
-      vfr[n] = row_frag(Vt, rbase, n, 0);
-    }
-    f32x16 s[QT], dp[QT];
+    for (int n = 0; n < PF; n++)
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+        kfr[n][kt] = row_frag(Kt, rbase, n, kt);
+        vfr[n][kt] = row_frag(Vt, rbase, n, kt);
+      }
+    f32x16 s[2], dp[2];
     FENCE();
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
 #pragma unroll
-      for (int qt = 0; qt < QT; qt++) {
+      for (int kt = 0; kt < 2; kt++) {
         if (ks == 0) {
-          s[qt] = mfma32(kfr[0], qf[qt][0], f32x16{0});
-          dp[qt] = mfma32(vfr[0], dof[qt][0], f32x16{0});
+          s[kt] = mfma32(kfr[0][kt], qf[0][0], f32x16{0});
+          dp[kt] = mfma32(vfr[0][kt], dof[0][0], f32x16{0});
         } else {
-          s[qt] = mfma32(kfr[ks % PF], qf[qt][ks], s[qt]);
-          dp[qt] = mfma32(vfr[ks % PF], dof[qt][ks], dp[qt]);
+          s[kt] = mfma32(kfr[ks % PF][kt], qf[0][ks], s[kt]);
+          dp[kt] = mfma32(vfr[ks % PF][kt], dof[0][ks], dp[kt]);
         }
       }
       if (ks + PF < KS) {
-        kfr[ks % PF] = row_frag(Kt, rbase, ks + PF, 0);
-        vfr[ks % PF] = row_frag(Vt, rbase, ks + PF, 0);
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+          kfr[ks % PF][kt] = row_frag(Kt, rbase, ks + PF, kt);
+          vfr[ks % PF][kt] = row_frag(Vt, rbase, ks + PF, kt);
+        }
       }
       FENCE();
     }
-    bf16x8 ifr[PF];
+    constexpr int IPF = 4;
+    bf16x8 ifr[IPF];
 #pragma unroll
-    for (int n = 0; n < PF; n++) ifr[n] = image_frag(Ki, ibase, n & 3, n >> 2, 0);
+    for (int n = 0; n < IPF; n++) ifr[n] = image_frag(Ki, ibase, n & 3, 0, 0);
     if (masked) {
 #pragma unroll
-      for (int qt = 0; qt < QT; qt++)
+      for (int kt = 0; kt < 2; kt++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
-          if (t * BN + acc_tile_row(r, g, 0) + 2 * kt > lim[qt]) s[qt][r] = -INFINITY;
+          if (t * BN + acc_tile_row(r, g, kt) > lim[0]) s[kt][r] = -INFINITY;
     }
-    bf16x8 dsf[QT][2];
+    bf16x8 dsf[2][2];
 #pragma unroll
-    for (int qt = 0; qt < QT; qt++)
+    for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const float pr = ody_exp2(fmaf(s[qt][r], c2, -lse2[qt]));
-        dsf[qt][r >> 3][r & 7] = (bf16)(pr * (dp[qt][r] - delta[qt]));
+        const float pr = ody_exp2(fmaf(s[kt][r], c2, -lse2[0]));
+        dsf[kt][r >> 3][r & 7] = (bf16)(pr * (dp[kt][r] - delta[0]));
       }
     FENCE();
 #pragma unroll
-    for (int n = 0; n < 8; n++) {
-      const int dt = n & 3, ss = n >> 2;
-#pragma unroll
-      for (int qt = 0; qt < QT; qt++) dq[qt][dt] = mfma32(ifr[n % PF], dsf[qt][ss], dq[qt][dt]);
-      if (n + PF < 8) ifr[n % PF] = image_frag(Ki, ibase, (n + PF) & 3, (n + PF) >> 2, 0);
+    for (int n = 0; n < 16; n++) {
+      const int dt = n & 3, ss = (n >> 2) & 1, kt = n >> 3;
+      dq[0][dt] = mfma32(ifr[n % IPF], dsf[kt][ss], dq[0][dt]);
+      if (n + IPF < 16) {
+        const int m = n + IPF;
+        ifr[n % IPF] = image_frag(Ki, ibase, m & 3, (m >> 2) & 1, m >> 3);
+      }
       FENCE();
     }
   };
@@ -185,12 +193,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
     __syncthreads();
     const bf16* st = ring + (t % 3) * STAGE;
     const bool dead = p.causal && t * BN > wq0 + 32 * QT - 1 + p.off;   // every key of the tile is after this wavefront's queries
-#pragma unroll 1
-    for (int kt = 0; kt < 2; kt++) {
-      // half of the loads of stage t+2 before each sub-tile (all at once they queue up at the memory pipeline)
-      if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, kt);
-      if (!dead) sub_tile(st, t, kt, t >= n_full);
-    }
+    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 0);
+    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 1);
+    if (!dead) tile(st, t, t >= n_full);
   }
 
 #pragma unroll
