@@ -146,7 +146,7 @@ def main():
     f_fwd, f_bwd = attn_flops(L, L, H, D)
     # algorithmic FLOPs per launch: the backward's 5 tile products are S, dP, dV, dK (in the
     # dK/dV kernel) and dQ (in the dQ kernel); the S and dP the dQ kernel recomputes are not counted
-    algo = {"attn_fwd_pipe": f_fwd, "attn_bwd_dkdv_pipe": f_bwd * 4 / 5, "attn_bwd_dq_pipe": f_bwd * 1 / 5}
+    algo = {"attn_fwd_w8": f_fwd, "attn_bwd_dkdv_pipe": f_bwd * 4 / 5, "attn_bwd_dq_pipe": f_bwd * 1 / 5}
     missing = [n for n in algo if n not in prof]
     if missing:
         raise SystemExit(f"bench.py: the library ran no kernel named {missing}; it reported {sorted(prof)}")

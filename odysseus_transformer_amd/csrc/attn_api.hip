@@ -1,6 +1,5 @@
 // extern "C" entry points for attention.
 #include <cmath>
-#include <cstdlib>
 #include "attn_params.h"
 
 namespace {
@@ -63,7 +62,6 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
                 workspace_bytes, need);
     ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
                 "ody_attn_fwd: workspace must be 256-byte aligned");
-    if (getenv("ODY_FWD_OLD")) return ody_launch_attn_fwd_pipe(p, workspace, st);
     return ody_launch_attn_fwd_w8(p, workspace, st);
   }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
@@ -72,7 +70,7 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
 
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
   if (B <= 0 || Lq <= 0 || Lk <= 0 || Hq <= 0 || Hkv <= 0) return 0;
-  if (dtype == ODY_BF16 && D == 128) return (ody_attn_fwd_pipe_workspace(B, Lq, Lk, Hq, Hkv) + 255) & ~(size_t)255;
+  if (dtype == ODY_BF16 && D == 128) return (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv) + 255) & ~(size_t)255;
   return 0;
 }
 

@@ -43,15 +43,12 @@ __device__ __forceinline__ BlockCoord ody_block_coord(int H, int B) {
 
 // Launchers (one per translation unit); each returns an ody_status.
 int ody_launch_attn_fwd_mfma(const AttnParams& p, int D, hipStream_t st);
-// head_dim 128 only; workspace of ody_attn_fwd_pipe_workspace(...) bytes
-int ody_launch_attn_fwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
 // transposed 64-row tile images of a (B, L, H, 128) bf16 matrix (attn_tile.h)
 size_t ody_attn_images_bytes(int B, int L, int H);
 // also zeroes `nflags` ints at `flags` (may be NULL)
 int ody_launch_attn_images(const void* src, const AttnStrides& s, int B, int L, int H, void* dst, int* flags,
                            int nflags, hipStream_t st);
-size_t ody_attn_fwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
-// the same with 8 wavefronts x 32 queries per block; same workspace layout
+// head_dim 128 only, 8 wavefronts x 32 queries per block; workspace of ody_attn_fwd_w8_workspace(...) bytes
 int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, hipStream_t st);
 size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
 // the online-rescaling forward kernel restricted to query blocks of `block` rows whose flag is set
