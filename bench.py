@@ -9,6 +9,7 @@ inputs, already resident in HBM).  `value` is the algorithmic TFLOP/s of that st
   roofline      the dominant kernel's algorithmic FLOP rate against the bf16 dense
                 MFMA peak, its duration measured with HIP events on the launch stream
   kernels       the same for every attention kernel of the step
+  mfma_sustained  what a loop of nothing but MFMAs sustains with constant and with random operands
   layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs,
                 RoPE, RMSNorm, SwiGLU) and the resulting tokens/s
   cpu_baseline  the CPU oracle timed on this host's cores on a bounded sample
@@ -61,6 +62,28 @@ def measured_traffic():
         return {}
     m = re.search(r"```json\s*(\{.*?\})\s*```", f.read_text(), re.S)
     return json.loads(m.group(1)) if m else {}
+
+
+def mfma_sustained(_lib, dev):
+    """What the matrix pipe sustains in a loop of nothing but MFMAs on register operands: with
+    constant operands (the published peak is reached) and with random ones (what real data allows)."""
+    import torch
+    blocks, iters = 512, 8000            # 8 wavefronts per CU; ~10 ms at the rates seen
+    sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    res = {}
+    g = torch.Generator().manual_seed(7)
+    for name, data in (("constant_operands", torch.ones(1 << 19)), ("random_operands", torch.randn(1 << 19, generator=g))):
+        ops_ = data.to(torch.bfloat16).to(dev)
+        for _ in range(2):
+            _lib.call("ody_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, 200, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.call("ody_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, iters, torch.cuda.current_stream().cuda_stream)
+        e1.record()
+        torch.cuda.synchronize()
+        res[name + "_tflops"] = round(blocks * 4 * iters * 16 * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+    return res
 
 
 def cpu_baseline():
@@ -179,6 +202,8 @@ def main():
         "kernels": kernels,
     }
 
+    # context for the roofline: the rate a register-only MFMA loop sustains on this box
+    out["mfma_sustained"] = mfma_sustained(_lib, dev)
     if not a.no_layer:
         out["layer"] = layer_share(ops, rn, dev, sec)
     if not a.no_cpu_baseline:

@@ -54,6 +54,14 @@ int ody_version(void);
 int ody_profile_enable(int on);
 int ody_profile_collect(char* out, size_t cap);
 
+/* Measurement aid (no counterpart in the reference): a loop of nothing but bf16 32x32x16 MFMAs on
+ * register operands taken from `operands` (at least 1 MiB of bf16 on the device), 4 wavefronts per
+ * block, 16 * iters MFMAs per wavefront, 32768 FLOP each.  What it sustains with the operand data
+ * of interest is the rate the matrix pipe can actually be driven at -- with random data well below
+ * the published peak, which only constant operands reach.  sink: blocks * 256 floats.
+ */
+int ody_mfma_probe(const void* operands, float* sink, int blocks, int iters, void* stream);
+
 /* ---- attention ---------------------------------------------------------
  * Replaces flash_attn_func(q, k, v, dropout_p=0, softmax_scale, causal) as
  * reached from decoder/odysseus.py:256-263 (via HF _flash_attention_forward),

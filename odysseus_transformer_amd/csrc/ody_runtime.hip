@@ -90,3 +90,46 @@ extern "C" int ody_profile_collect(char* out, size_t cap) {
   memcpy(out, txt.c_str(), txt.size() + 1);
   return ODY_OK;
 }
+
+// ---------------------------------------------------------------------------
+// MFMA-only loop on register operands: the sustained rate of the matrix pipe for given operand data
+// ---------------------------------------------------------------------------
+namespace {
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const bf16x8* __restrict__ in, float* __restrict__ sink,
+                                                         int iters) {
+  const int tid = blockIdx.x * 256 + threadIdx.x;
+  bf16x8 a[4], b[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    a[j] = in[(tid * 8 + j) & 0xffff];
+    b[j] = in[(tid * 8 + 4 + j) & 0xffff];
+  }
+  f32x16 c[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[j][r] = 0.f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int u = 0; u < 4; u++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) c[j] = mfma32(a[(u + j) & 3], b[u], c[j]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) s += c[j][r];
+  sink[tid] = s;
+}
+}  // namespace
+
+extern "C" int ody_mfma_probe(const void* operands, float* sink, int blocks, int iters, void* stream) {
+  ODY_REQUIRE(operands && sink, ODY_ERR_NULL, "ody_mfma_probe: NULL pointer");
+  ODY_REQUIRE(blocks > 0 && iters > 0, ODY_ERR_BAD_SHAPE, "ody_mfma_probe: blocks=%d iters=%d", blocks, iters);
+  ODY_REQUIRE(ody_aligned16(operands), ODY_ERR_MISALIGNED, "ody_mfma_probe: operands must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  ODY_LAUNCH("mfma_probe", st, mfma_probe_kernel, dim3(blocks), dim3(256), 0, static_cast<const bf16x8*>(operands), sink,
+             iters);
+  return ody_check_launch("mfma_probe");
+}
