@@ -259,17 +259,25 @@ __global__ __launch_bounds__(128) void attn_bwd_stats_kernel(const AttnParams p,
       bf16x8{hi, mid, lo, z, z, z, z, z};
 }
 
+//
+// SPLIT = false: a block owns 256 keys of one kv head and walks all query heads of its group.
+// SPLIT = true (grouped-query attention): a block owns 256 keys for ONE query head and writes
+// fp32 partial dK / dV to `part`, which attn_bwd_group_sum_kernel adds up over the group.  With few
+// kv heads this is what gives the chip enough, and evenly sized, blocks.
+template <bool SPLIT>
 __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
                                                                          const bf16* __restrict__ qimg,
                                                                          const bf16* __restrict__ doimg,
-                                                                         const bf16* __restrict__ stats) {
+                                                                         const bf16* __restrict__ stats,
+                                                                         float* __restrict__ part) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][KV_STAGE]
 
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
             i = lane & 31;
-  const BlockCoord bc = ody_block_coord(p.Hkv, p.B);   // rank 0 = first key block = most query tiles
-  const int hk = bc.h, b = bc.b;
+  const BlockCoord bc = ody_block_coord(SPLIT ? p.Hq : p.Hkv, p.B);   // rank 0 = first key block = most query tiles
+  const int hk = SPLIT ? bc.h / p.group : bc.h, b = bc.b;
+  const int h_first = SPLIT ? bc.h : hk * p.group, n_heads = SPLIT ? 1 : p.group;   // query heads this block walks
   const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
   const int q_tiles = (p.Lq + KV_BQ - 1) / KV_BQ;
   simd_stagger(tid);
@@ -297,13 +305,13 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 
   const int t_begin = p.causal ? max(0, n0 - p.off) / KV_BQ : 0;   // first query tile that sees a key of this block
   const int ntq = max(0, q_tiles - t_begin);
-  const int total = ntq * p.group;   // flattened (head of the group, query tile)
+  const int total = ntq * n_heads;   // flattened (query head, query tile)
   const float c2 = p.scale_log2e;
 
   // Direct loads of one stage: uniform base pointers plus 32-bit per-lane offsets that are
   // recomputed from the lane id every time (cheaper than keeping them in registers here).
   auto load_stage = [&](bf16* st, int it, int j) {   // j = 0, 1: the two halves of the stage's loads
-    const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = hk * p.group + hg;
+    const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = h_first + hg;
     const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h + (int64_t)t * KV_BQ * p.sq.l;
     const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h + (int64_t)t * KV_BQ * p.sdo.l;
     const int64_t tile_id = ((int64_t)b * p.Hq + h) * q_tiles + t;
@@ -417,7 +425,23 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     }
   }
 
-  if (key < p.Lk) {
+  if (SPLIT) {
+    if (key < p.Lk) {
+      // part: [dK | dV][batch][query head][key][D] fp32, unscaled
+      float* pk = part + (((int64_t)b * p.Hq + h_first) * p.Lk + key) * D;
+      float* pv = pk + (int64_t)p.B * p.Hq * p.Lk * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          f32x4 wk, wv;
+#pragma unroll
+          for (int e = 0; e < 4; e++) wk[e] = dk[dt][4 * a + e], wv[e] = dv[dt][4 * a + e];
+          *reinterpret_cast<f32x4*>(pk + 32 * dt + 8 * a + 4 * g) = wk;
+          *reinterpret_cast<f32x4*>(pv + 32 * dt + 8 * a + 4 * g) = wv;
+        }
+    }
+  } else if (key < p.Lk) {
     bf16* dkp = static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l;
     bf16* dvp = static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l;
 #pragma unroll
@@ -436,14 +460,42 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   }
 }
 
+// dK, dV of a kv head = sum of the fp32 partials of its query heads; one thread per 4 elements
+__global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParams p, const float* __restrict__ part) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;           // over B * Hkv * Lk * D / 4
+  const int64_t total = (int64_t)p.B * p.Hkv * p.Lk * (D / 4);
+  if (idx >= total) return;
+  const int d4 = idx % (D / 4);
+  const int key = (idx / (D / 4)) % p.Lk;
+  const int hk = (idx / ((int64_t)(D / 4) * p.Lk)) % p.Hkv;
+  const int b = idx / ((int64_t)(D / 4) * p.Lk * p.Hkv);
+  const int64_t plane = (int64_t)p.B * p.Hq * p.Lk * D;
+  f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = sk;
+  for (int hg = 0; hg < p.group; hg++) {
+    const float* src = part + (((int64_t)b * p.Hq + hk * p.group + hg) * p.Lk + key) * D + 4 * d4;
+    sk += *reinterpret_cast<const f32x4*>(src);
+    sv += *reinterpret_cast<const f32x4*>(src + plane);
+  }
+  bf16x4 wk, wv;
+#pragma unroll
+  for (int e = 0; e < 4; e++) wk[e] = (bf16)(sk[e] * p.scale), wv[e] = (bf16)sv[e];
+  *reinterpret_cast<bf16x4*>(static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l + 4 * d4) = wk;
+  *reinterpret_cast<bf16x4*>(static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l + 4 * d4) = wv;
+}
+
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+inline size_t group_partials_bytes(int B, int Lk, int Hq, int Hkv) {
+  return Hq == Hkv ? 0 : align256((size_t)2 * B * Hq * Lk * D * sizeof(float));
+}
 
 }  // namespace
 
-// workspace after delta: the transposed images of K, Q and dO, and the per-tile start values
+// workspace after delta: the transposed images of K, Q and dO, the per-tile start values and, for
+// grouped-query attention, the fp32 partial dK / dV of every query head
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
   return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq)) +
-         align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16));
+         align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)) +
+         group_partials_bytes(B, Lk, Hq, Hkv);
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
@@ -453,7 +505,9 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess) {
       ody_set_error("attn_bwd: hipFuncSetAttribute failed");
       return ODY_ERR_LAUNCH;
@@ -474,9 +528,23 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
   if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
   if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
-  dim3 gk(((p.Lk + KV_BN - 1) / KV_BN) * p.Hkv * p.B);
-  ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel, gk, dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats);
-  if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
+  const int key_blocks = (p.Lk + KV_BN - 1) / KV_BN;
+  if (p.group == 1) {
+    ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<false>, dim3(key_blocks * p.Hkv * p.B),
+               dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
+    if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
+  } else {
+    float* part = reinterpret_cast<float*>(
+        reinterpret_cast<unsigned char*>(stats) +
+        align256((size_t)p.B * p.Hq * ((p.Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)));
+    ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<true>, dim3(key_blocks * p.Hq * p.B),
+               dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
+    if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
+    const int64_t n4 = (int64_t)p.B * p.Hkv * p.Lk * (D / 4);
+    ODY_LAUNCH("attn_bwd_group_sum", st, attn_bwd_group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, p,
+               part);
+    if ((rc = ody_check_launch("attn_bwd_group_sum"))) return rc;
+  }
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");
