@@ -136,11 +136,15 @@ int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk, const flo
  *                                                           utils/linear_zero3.py:74
  * bias (N) of `dtype` or NULL is added to every row (utils/linear_tpsp.py:175-176).
  * If accumulate != 0, C += result (C read in `dtype`, added in fp32).
+ * workspace (optional, 16-byte aligned): with ody_gemm_workspace_bytes(...) > 0 bytes of it a product
+ * with a long K and few output tiles (a weight gradient) is computed over several ranges of K at once
+ * and summed in fp32; without it (NULL / too small) the same result comes from one pass over K.
  */
 enum ody_gemm_op { ODY_GEMM_NT = 0, ODY_GEMM_NN = 1, ODY_GEMM_TN = 2 };
+size_t ody_gemm_workspace_bytes(int op, int M, int N, int K, int dtype);
 int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias,
              int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
-             int accumulate, int dtype, void* stream);
+             int accumulate, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ---- SwiGLU -------------------------------------------------------------
  * decoder/odysseus.py:293-295: a1, a3 = gate_up.chunk(2, -1); h = silu(a1) * a3.

@@ -28,7 +28,8 @@ SIGNATURES = {
     "ody_attn_bwd_workspace_bytes": (_sz, [_i] * 7),
     "ody_attn_bwd": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p]),
     "ody_lse_merge": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i, _p]),
-    "ody_gemm": (_i, [_i] + [_p] * 4 + [_i] * 3 + [_i64] * 3 + [_i, _i, _p]),
+    "ody_gemm_workspace_bytes": (_sz, [_i] * 5),
+    "ody_gemm": (_i, [_i] + [_p] * 4 + [_i] * 3 + [_i64] * 3 + [_i, _i, _p, _sz, _p]),
     "ody_swiglu_fwd": (_i, [_p, _p, _i, _i, _i64, _i64, _i, _p]),
     "ody_swiglu_bwd": (_i, [_p, _p, _p, _i, _i, _i64, _i64, _i64, _i, _p]),
     "ody_rmsnorm_fwd": (_i, [_p] * 4 + [_i, _i, _f, _i, _p]),

@@ -76,11 +76,16 @@ struct OperandTile {
 // reads of the next k-step.
 #define GEMM_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-template <int WM, int WN, bool A_KC, bool B_KC>
+//
+// SPLITK: blockIdx.y selects one of gridDim.y ranges of K slabs; the block writes its fp32 partial tile to
+// part[blockIdx.y][M][N] and gemm_splitk_sum_kernel adds the ranges up (bias, C += and the rounding happen
+// there).  For products with a long K and few output tiles (weight gradients) this is what fills the chip.
+template <int WM, int WN, bool A_KC, bool B_KC, bool SPLITK>
 __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
                                                              bf16* __restrict__ C, const bf16* __restrict__ bias,
                                                              int M, int N, int K, int64_t lda, int64_t ldb,
-                                                             int64_t ldc, int accumulate, int tiles_m, int tiles_n) {
+                                                             int64_t ldc, int accumulate, int tiles_m, int tiles_n,
+                                                             float* __restrict__ part) {
   constexpr int TM = 64 * WM, TN = 64 * WN;
   typedef OperandTile<TM, A_KC> TA;
   typedef OperandTile<TN, B_KC> TB;
@@ -122,8 +127,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     b_off0 = (unsigned)((tid / (TN / 8)) * ldb + (tid % (TN / 8)) * 8); b_step = (256 / (TN / 8)) * ldb; b_slab = BK * ldb;
     b_lds0 = (tid / (TN / 8)) * TB::PITCH + (tid % (TN / 8)) * 8; b_lstep = (256 / (TN / 8)) * TB::PITCH;
   }
-  const bf16* Abase = A_KC ? A + (int64_t)m0 * lda : A + m0;   // first element of the tile's slab 0
-  const bf16* Bbase = B_KC ? B + (int64_t)n0 * ldb : B + n0;
+  // this block's range of K slabs
+  int nk = K / BK, kt0 = 0;
+  if (SPLITK) {
+    const int per = (nk + (int)gridDim.y - 1) / (int)gridDim.y;
+    kt0 = blockIdx.y * per;
+    nk = max(0, min(nk - kt0, per));
+  }
+  const bf16* Abase = (A_KC ? A + (int64_t)m0 * lda : A + m0) + (int64_t)kt0 * a_slab;   // first element of the first slab
+  const bf16* Bbase = (B_KC ? B + (int64_t)n0 * ldb : B + n0) + (int64_t)kt0 * b_slab;
 
   f32x16 acc[WM][WN];
 #pragma unroll
@@ -143,7 +155,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
   auto sstore_a = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(As + buf * TA::ELEMS + a_lds0 + j * a_lstep) = ra[j]; };
   auto sstore_b = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(Bs + buf * TB::ELEMS + b_lds0 + j * b_lstep) = rb[j]; };
 
-  const int nk = K / BK;
+  if (nk > 0) {
 #pragma unroll
   for (int j = 0; j < CA; j++) gload_a(0, j);
 #pragma unroll
@@ -158,6 +170,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     for (int j = 0; j < CA; j++) gload_a(k1, j);
 #pragma unroll
     for (int j = 0; j < CB; j++) gload_b(k1, j);
+  }
   }
   __syncthreads();
 
@@ -207,6 +220,33 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
   // Epilogue.  Lane (g, i) holds column m = i and rows n = 8*(r/4) + 4g + r%4 of each 32 x 32 tile,
   // i.e. 8-byte pieces of 32 different rows of C.  Unless C is accumulated into, the tiles go
   // through LDS (free by now) one 32-row band at a time and leave as 16-byte pieces of whole rows.
+  if (SPLITK) {
+    // fp32 partial tile, through LDS like below: 32-row bands, 16-byte pieces of whole rows
+    constexpr int EPF = 32 * WN + 4;
+    float* band = reinterpret_cast<float*>(smem_raw) + wave * 32 * EPF;
+    static_assert(4 * 32 * EPF * 2 <= 2 * (TA::ELEMS + TB::ELEMS), "the fp32 bands fit in the operand buffers");
+    float* dst0 = part + ((int64_t)blockIdx.y * M + m0) * N + n0 + 32 * wn * WN;
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          *reinterpret_cast<f32x4*>(band + i * EPF + 32 * b + 8 * q + 4 * g) = v;
+        }
+      constexpr int CPR = 32 * WN / 4, RPP = 64 / CPR;                  // 16-byte chunks per row, rows per pass
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const f32x4 v = *reinterpret_cast<const f32x4*>(band + row * EPF + 4 * c);
+        *reinterpret_cast<f32x4*>(dst0 + (int64_t)(32 * (wm * WM + a) + row) * N + 4 * c) = v;
+      }
+    }
+    return;
+  }
   if (!accumulate) {
     constexpr int EP = 32 * WN + 8;                                     // band pitch in elements
     bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;   // 32 rows x (32 * WN) columns per wavefront
@@ -380,19 +420,62 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__
   }
 }
 
+// C = sum over the K ranges of the fp32 partial tiles (+ bias, + C), rounded once; 4 elements per thread
+__global__ __launch_bounds__(256) void gemm_splitk_sum_kernel(const float* __restrict__ part, int splits,
+                                                              bf16* __restrict__ C, const bf16* __restrict__ bias, int M,
+                                                              int N, int64_t ldc, int accumulate) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, total = (int64_t)M * (N / 4);
+  if (idx >= total) return;
+  const int m = idx / (N / 4), n = (idx % (N / 4)) * 4;
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < splits; s++) v += *reinterpret_cast<const f32x4*>(part + ((int64_t)s * M + m) * N + n);
+  if (bias) {
+    const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] += (float)bv[e];
+  }
+  bf16* dst = C + (int64_t)m * ldc + n;
+  if (accumulate) {
+    const bf16x4 old = *reinterpret_cast<const bf16x4*>(dst);
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] += (float)old[e];
+  }
+  bf16x4 w;
+#pragma unroll
+  for (int e = 0; e < 4; e++) w[e] = (bf16)v[e];
+  *reinterpret_cast<bf16x4*>(dst) = w;
+}
+
+// Number of K ranges for a product of full 256 x 256 tiles: only where the tiles alone would leave most
+// of the chip idle, and every range keeps at least 8 slabs.
+int splitk_plan(int M, int N, int K) {
+  if (M % 256 || N % 256 || K % BK) return 1;
+  const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+  const int nk = K / BK;
+  if (tiles > 128) return 1;
+  int splits = (int)(512 / tiles);
+  if (splits > 8) splits = 8;
+  if (splits > nk / 8) splits = nk / 8;
+  return splits < 2 ? 1 : splits;
+}
+
 template <int WM, int WN, bool A_KC, bool B_KC>
 int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, int N, int K, int64_t lda, int64_t ldb,
-                int64_t ldc, int accumulate, hipStream_t st) {
+                int64_t ldc, int accumulate, float* part, int splits, hipStream_t st) {
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr size_t smem = 2 * sizeof(bf16) * (OperandTile<TM, A_KC>::ELEMS + OperandTile<TN, B_KC>::ELEMS);
   static bool attr_set = false;
   auto kern = &gemm_bf16_kernel<WM, WN, A_KC, B_KC>;
-  auto fast = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC>;
+  auto fast = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC, false>;
+  auto fastk = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC, true>;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e == hipSuccess)
       e = hipFuncSetAttribute(reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)smem);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(fastk), hipFuncAttributeMaxDynamicSharedMemorySize,
                               (int)smem);
     if (e != hipSuccess) {
       ody_set_error("ody_gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
@@ -407,9 +490,19 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
                         ody_aligned16(C) && ldc % 8 == 0 &&
                         (int64_t)TN * ldb < (1ll << 31) && (int64_t)BK * lda < (1ll << 31) &&
                         (int64_t)BK * ldb < (1ll << 31);
+  if (interior && splits > 1) {
+    ODY_LAUNCH(name, st, fastk, dim3(tiles_m * tiles_n, splits), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
+               accumulate, tiles_m, tiles_n, part);
+    int rc = ody_check_launch("gemm_bf16");
+    if (rc) return rc;
+    const int64_t n4 = (int64_t)M * (N / 4);
+    ODY_LAUNCH("gemm_splitk_sum", st, gemm_splitk_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, part,
+               splits, C, bias, M, N, ldc, accumulate);
+    return ody_check_launch("gemm_splitk_sum");
+  }
   if (interior) {
     ODY_LAUNCH(name, st, fast, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
-               accumulate, tiles_m, tiles_n);
+               accumulate, tiles_m, tiles_n, nullptr);
     return ody_check_launch("gemm_bf16");
   }
   ODY_LAUNCH(name, st, kern, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
@@ -419,11 +512,18 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
 
 template <bool A_KC, bool B_KC>
 int dispatch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, int N, int K, int64_t lda,
-                  int64_t ldb, int64_t ldc, int accumulate, hipStream_t st) {
+                  int64_t ldb, int64_t ldc, int accumulate, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  // long K, few output tiles, and the caller brought the workspace: 256 x 256 tiles over ranges of K
+  const int splits = splitk_plan(M, N, K);
+  if (splits > 1 && workspace && workspace_bytes >= (size_t)splits * M * N * sizeof(float) && ody_aligned16(workspace) &&
+      ody_aligned16(C) && ldc % 8 == 0)
+    return launch_bf16<4, 4, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate,
+                                         static_cast<float*>(workspace), splits, st);
   // large problems: 256 x 256 tiles; otherwise 128 x 128 so that the grid still covers the chip
   const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (big_tiles >= 192) return launch_bf16<4, 4, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, st);
-  return launch_bf16<2, 2, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, st);
+  if (big_tiles >= 192)
+    return launch_bf16<4, 4, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, nullptr, 1, st);
+  return launch_bf16<2, 2, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, nullptr, 1, st);
 }
 
 // ------------------------------------------------------------------ fp32 SIMT
@@ -482,8 +582,16 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 
 }  // namespace
 
+extern "C" size_t ody_gemm_workspace_bytes(int op, int M, int N, int K, int dtype) {
+  (void)op;
+  if (dtype != ODY_BF16 || M <= 0 || N <= 0 || K <= 0) return 0;
+  const int splits = splitk_plan(M, N, K);
+  return splits > 1 ? (size_t)splits * M * N * sizeof(float) : 0;
+}
+
 extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias, int M, int N, int K,
-                        int64_t lda, int64_t ldb, int64_t ldc, int accumulate, int dtype, void* stream) {
+                        int64_t lda, int64_t ldb, int64_t ldc, int accumulate, int dtype, void* workspace,
+                        size_t workspace_bytes, void* stream) {
   ODY_REQUIRE(A && B && C, ODY_ERR_NULL, "ody_gemm: NULL pointer");
   ODY_REQUIRE(M > 0 && N > 0 && K > 0, ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d N=%d K=%d", M, N, K);
   ODY_REQUIRE(op == ODY_GEMM_NT || op == ODY_GEMM_NN || op == ODY_GEMM_TN, ODY_ERR_UNSUPPORTED, "ody_gemm: op %d", op);
@@ -514,7 +622,9 @@ extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const voi
               "(M=%d N=%d K=%d op=%d)", M, N, K, op);
   const bf16 *a = (const bf16*)A, *b = (const bf16*)B, *bs = (const bf16*)bias;
   bf16* c = (bf16*)C;
-  if (op == ODY_GEMM_NT) return dispatch_bf16<true, true>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
-  if (op == ODY_GEMM_NN) return dispatch_bf16<true, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
-  return dispatch_bf16<false, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, st);
+  if (op == ODY_GEMM_NT)
+    return dispatch_bf16<true, true>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+  if (op == ODY_GEMM_NN)
+    return dispatch_bf16<true, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+  return dispatch_bf16<false, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
 }

@@ -128,9 +128,11 @@ def gemm(op: int, a, b, bias=None, out=None, accumulate: bool = False):
         if accumulate:
             raise ValueError("accumulate needs an existing out")
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    ws_bytes = _lib.load().ody_gemm_workspace_bytes(op, M, N, K, _dt(a))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     _lib.call("ody_gemm", op, a.data_ptr(), b.data_ptr(), out.data_ptr(), 0 if bias is None else bias.data_ptr(),
               M, N, K, _rowmajor2d(a, "a"), _rowmajor2d(b, "b"), _rowmajor2d(out, "out"),
-              int(accumulate), _dt(a), _stream())
+              int(accumulate), _dt(a), ws.data_ptr() if ws is not None else 0, ws_bytes, _stream())
     return out
 
 

@@ -34,7 +34,7 @@ def test_validation_returns_codes_without_a_gpu():
     lib = _lib.load()
     # bad shapes / NULL pointers are rejected before anything touches the device
     with pytest.raises(_lib.OdysseusHipError) as e:
-        _lib.call("ody_gemm", 0, 0, 0, 0, 0, 8, 8, 8, 8, 8, 8, 0, 0, 0)
+        _lib.call("ody_gemm", 0, 0, 0, 0, 0, 8, 8, 8, 8, 8, 8, 0, 0, 0, 0, 0)
     assert e.value.code == -4 and "NULL" in e.value.msg
     with pytest.raises(_lib.OdysseusHipError) as e:
         _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 3, 2, 128, *([128] * 12), 1.0, 1, 0, 0, 0, 0)
