@@ -172,3 +172,14 @@ def test_functional_linear_signature_and_dead_branches():
     with pytest.raises(AssertionError, match="Batch size should be 1"):
         lt.linear_with_grad_accumulation_and_async_allreduce(torch.zeros(2, 3, 8), torch.zeros(4, 8), None, False,
                                                              False, True)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU only: `bench.py --gpus N` with N above 1 exits with a message that says so."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
