@@ -135,3 +135,38 @@ def test_attention_errors(dev):
         ops.attn_fwd(q, q, q)
     with pytest.raises(RuntimeError):              # CPU tensors are refused, no fallback
         ops.attn_fwd(q.cpu(), q.cpu(), q.cpu())
+
+
+def _random_cases(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    cases = []
+    for _ in range(n):
+        hkv = [1, 2, 4][r(0, 2)]
+        grp = [1, 2, 4][r(0, 2)]
+        lq = [r(1, 96), r(97, 400), r(401, 1100)][r(0, 2)]
+        kind = r(0, 3)                       # 0/1: square causal, 2: causal with more keys, 3: full block
+        lk = lq if kind < 2 else lq + r(1, 500) if kind == 2 else r(1, 900)
+        cases.append((r(1, 2), lq, lk, hkv * grp, hkv, kind != 3))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(36, 2024), ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d" % c)
+def test_attention_random_shapes(case, dev):
+    """Ragged lengths on both sides of every tile size (32, 64, 256), key offsets, group sizes 1/2/4."""
+    from odysseus_transformer_amd import ops
+    B, Lq, Lk, Hq, Hkv, causal = case
+    print(f"case={case}", flush=True)
+    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, 128, torch.bfloat16, seed=Lq * 7 + Lk)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float(),
+                                                  causal=causal)
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
+    dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal)
+    floor = 1.0 if Lk == 1 else 1e-3
+    assert rel_err(o, o_ref) <= TOL_BF16
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    assert rel_err(dq, dq_ref, floor) <= TOL_BF16, "dq"
+    assert rel_err(dk, dk_ref, floor) <= TOL_BF16, "dk"
+    assert rel_err(dv, dv_ref) <= TOL_BF16, "dv"
