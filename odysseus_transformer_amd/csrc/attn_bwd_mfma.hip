@@ -364,27 +364,8 @@ int launch(const AttnParams& p, hipStream_t st) {
 
 }  // namespace
 
-// the dK/dV kernel alone (head_dim 128), for the launcher that pairs it with the dQ kernel of attn_bwd_pipe.hip
-int ody_launch_attn_bwd_dkdv_mfma(const AttnParams& p, hipStream_t st) {
-  constexpr int D = 128;
-  constexpr size_t smem_kv = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16) + 2 * 2 * 64 * sizeof(float);
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess) {
-      ody_set_error("attn_bwd: hipFuncSetAttribute failed");
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
-  dim3 gk(((p.Lk + 127) / 128) * p.Hkv * p.B);
-  ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
-  return ody_check_launch("attn_bwd_dkdv");
-}
-
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 128) return launch<128>(p, st);
-  if (D == 64) return launch<64>(p, st);
-  ody_set_error("attn_bwd: head_dim %d not built (64, 128)", D);
+  if (D == 64) return launch<64>(p, st);   // head_dim 128 has its own kernels (attn_bwd_pipe.hip)
+  ody_set_error("attn_bwd: head_dim %d not built here (64)", D);
   return ODY_ERR_UNSUPPORTED;
 }

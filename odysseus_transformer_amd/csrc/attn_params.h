@@ -57,7 +57,6 @@ int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int 
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st);
-int ody_launch_attn_bwd_dkdv_mfma(const AttnParams& p, hipStream_t st);   // head_dim 128
 int ody_launch_attn_fwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);
 int ody_launch_attn_bwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);
 int ody_launch_attn_delta(const AttnParams& p, int D, int dtype, hipStream_t st);
