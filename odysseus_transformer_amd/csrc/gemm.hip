@@ -70,10 +70,10 @@ struct OperandTile {
 // general kernel below, but the traffic of the next slabs is spread over the MFMA stream
 // instead of being issued in bursts: a wavefront is held up while the memory pipeline accepts
 // its loads (64 bytes per clock per CU) and while the LDS takes its writes, and with one
-// wavefront per SIMD the matrix pipe idles meanwhile.  Per 16-MFMA k-step the wavefront issues
-// a quarter of the global loads of slab kt+2 (into one of two register sets), a quarter of the
-// LDS writes of slab kt+1 (from the other set, loaded one iteration earlier) and the fragment
-// reads of the next k-step.
+// wavefront per SIMD the matrix pipe idles meanwhile.  Per 16-MFMA k-step the wavefront writes
+// a quarter of its staging registers (slab kt+1, loaded one iteration earlier) to the other LDS
+// buffer, refills them at once with their part of slab kt+2, and reads the fragments of the next
+// k-step.
 #define GEMM_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 //
@@ -526,6 +526,34 @@ int dispatch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M
   return launch_bf16<2, 2, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, nullptr, 1, st);
 }
 
+// One bf16 product.  A ragged M or N is cut into a main part of whole tiles, which takes the fast
+// kernel, and an edge strip on the right and at the bottom for the general kernel.
+int gemm_bf16(int op, const bf16* a, const bf16* b, bf16* c, const bf16* bias, int M, int N, int K, int64_t lda,
+              int64_t ldb, int64_t ldc, int accumulate, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  const int64_t big_tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  const int tile = big_tiles >= 192 ? 256 : 128;
+  const int M0 = M / tile * tile, N0 = N / tile * tile;
+  if (K % BK == 0 && M0 > 0 && N0 > 0 && (M0 < M || N0 < N)) {
+    int rc = gemm_bf16(op, a, b, c, bias, M0, N0, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+    if (rc) return rc;
+    if (N0 < N) {   // right strip: every row, columns [N0, N)
+      const bf16* b1 = (op == ODY_GEMM_NT) ? b + (int64_t)N0 * ldb : b + N0;
+      rc = gemm_bf16(op, a, b1, c + N0, bias ? bias + N0 : nullptr, M, N - N0, K, lda, ldb, ldc, accumulate, nullptr, 0, st);
+      if (rc) return rc;
+    }
+    if (M0 < M) {   // bottom strip: rows [M0, M), columns [0, N0)
+      const bf16* a1 = (op == ODY_GEMM_TN) ? a + M0 : a + (int64_t)M0 * lda;
+      rc = gemm_bf16(op, a1, b, c + (int64_t)M0 * ldc, bias, M - M0, N0, K, lda, ldb, ldc, accumulate, nullptr, 0, st);
+    }
+    return rc;
+  }
+  if (op == ODY_GEMM_NT)
+    return dispatch_bf16<true, true>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+  if (op == ODY_GEMM_NN)
+    return dispatch_bf16<true, false>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+  return dispatch_bf16<false, false>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+}
+
 // ------------------------------------------------------------------ fp32 SIMT
 // A(m, k) = A[m * sam + k * sak], B(k, n) = B[k * sbk + n * sbn]
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
@@ -620,11 +648,6 @@ extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const voi
   ODY_REQUIRE(N % 8 == 0 && a_cols % 8 == 0 && b_cols % 8 == 0, ODY_ERR_UNSUPPORTED,
               "ody_gemm: bf16 path needs N and the contiguous extents of A and B to be multiples of 8 "
               "(M=%d N=%d K=%d op=%d)", M, N, K, op);
-  const bf16 *a = (const bf16*)A, *b = (const bf16*)B, *bs = (const bf16*)bias;
-  bf16* c = (bf16*)C;
-  if (op == ODY_GEMM_NT)
-    return dispatch_bf16<true, true>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
-  if (op == ODY_GEMM_NN)
-    return dispatch_bf16<true, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
-  return dispatch_bf16<false, false>(a, b, c, bs, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
+  return gemm_bf16(op, (const bf16*)A, (const bf16*)B, (bf16*)C, (const bf16*)bias, M, N, K, lda, ldb, ldc, accumulate,
+                   workspace, workspace_bytes, st);
 }

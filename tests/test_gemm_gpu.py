@@ -18,6 +18,8 @@ SHAPES = [
     (520, 2752, 512),      # gate_up of the fp32 configuration, ragged M
     (1024, 768, 4096),
     (4096, 4096, 512),     # enough tiles for the 256 x 256 kernel
+    (1000, 1096, 256),     # whole tiles plus a ragged strip on the right and at the bottom
+    (4104, 3848, 128),     # the same with 256 x 256 tiles
 ]
 
 
