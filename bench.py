@@ -88,13 +88,13 @@ def mfma_sustained(_lib, dev):
 
 def cpu_baseline():
     """The oracle (plain PyTorch, fp32) on the host cores: causal attention fwd+bwd at
-    4 heads x 128, L = 8192 -- 1/16 of the FLOPs of one benchmark step."""
+    4 heads x 128, L = 16384 -- 1/4 of the FLOPs of one benchmark step (tens of core-seconds)."""
     import torch
     sys.path.insert(0, str(ROOT / "oracle"))
     import odysseus_oracle as oracle
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    Ls = 8192
+    Ls = 16384
     g = torch.Generator().manual_seed(2000)
     q, k, v, do = (torch.randn(1, Ls, H, D, generator=g) for _ in range(4))
     t0 = time.perf_counter()
@@ -103,7 +103,7 @@ def cpu_baseline():
     dt = time.perf_counter() - t0
     f, b = attn_flops(Ls, Ls, H, D)
     return {"value": (f + b) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"causal attention fwd+bwd, {H} heads x {D}, L={Ls} (1/16 of the step's FLOPs), fp32, "
+            "sample": f"causal attention fwd+bwd, {H} heads x {D}, L={Ls} (1/4 of the step's FLOPs), fp32, "
                       f"{dt:.2f} s wall"}
 
 

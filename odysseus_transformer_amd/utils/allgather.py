@@ -1,9 +1,12 @@
-"""Sequence all-gather of a batch-1 activation (utils/allgather.py:4-10 of the reference)."""
-from .linear_tpsp import allgather_along_first_dim_from_model_parallel_region
+"""`allgather_bsz1` (utils/allgather.py:4-10 of the reference): the sequence all-gather of a
+(1, L/N, h) activation into (1, L, h).  The collective works on the leading dimension, so the
+batch axis of extent 1 is what gets gathered and the result is re-viewed with it in front."""
+from . import linear_tpsp as _tpsp
 
 
 def allgather_bsz1(x):
-    bsz, seqlen, h = x.shape
-    assert bsz == 1, f"Batch size {bsz} must be 1 for allgather_bsz1"
-    x = allgather_along_first_dim_from_model_parallel_region(x)
-    return x.view(bsz, -1, h)
+    if x.dim() != 3 or x.shape[0] != 1:
+        raise AssertionError(f"allgather_bsz1 takes a (1, seq, hidden) tensor, got {tuple(x.shape)}")
+    hidden = x.shape[2]
+    gathered = _tpsp.allgather_along_first_dim_from_model_parallel_region(x)
+    return gathered.reshape(1, -1, hidden)
