@@ -1,17 +1,19 @@
-// Flash-attention backward, head_dim 128, bf16: the dQ kernel on the tile machinery of
-// attn_tile.h -- direct global->LDS loads into a three-deep ring, 16-byte LDS reads only
-// (K^T comes from the transposed images a pre-pass writes), fenced slots that keep LDS
-// operand prefetch and MFMAs interleaved.  Query-stationary, 8 wavefronts x 32 queries
-// (two wavefronts per SIMD overlap each other's matrix and vector phases), lane = query
-// column, so lse and delta are per-lane scalars:
+// Flash-attention backward, head_dim 128, bf16, on the tile machinery of attn_tile.h: direct
+// global->LDS loads into a ring of stages, 16-byte LDS reads only (an operand that a product
+// contracts over its row index comes from the transposed images a pre-pass writes), fenced slots
+// that keep LDS operand prefetch and MFMAs interleaved, 8 wavefronts per block = two per SIMD,
+// which overlap each other's matrix and vector phases.  Two kernels, no atomics: both recompute S
+// from the saved log-sum-exp, and each owns its outputs.
+//
+// dQ kernel -- query-stationary, 32 queries per wavefront, lane = query column, so lse and delta
+// are per-lane scalars; a three-deep ring of {K tile, V tile, K^T image}:
 //
 //      S^T = K Q^T            A: K rows (LDS)        B: Q^T (registers)
 //      dP^T = V dO^T          A: V rows (LDS)        B: dO^T (registers)
 //      dS^T = exp2(S^T c - lse) * (dP^T - delta)
 //      dQ^T += K^T dS^T       A: K^T image (LDS)     B: dS^T = accumulator layout
 //
-// The dK/dV half of the backward is the key-stationary kernel of attn_bwd_mfma.hip.  No
-// atomics anywhere: both kernels recompute S, and each owns its outputs.
+// dK/dV kernel -- key-stationary, 32 keys per wavefront (described where it is defined).
 #include <type_traits>
 #include "attn_params.h"
 #include "attn_tile.h"
