@@ -15,8 +15,7 @@ int check_common(const char* who, int B, int Lq, int Lk, int Hq, int Hkv, int D,
   return ODY_OK;
 }
 
-// The MFMA kernels move 16-byte vectors: pointers 16-byte aligned, strides multiples of 8 elements.
-// The fp32 kernels use scalar accesses except for the delta pre-pass (16-byte vectors of 4 floats).
+// All kernels move 16-byte vectors: pointers 16-byte aligned, strides multiples of 8 (bf16) or 4 (fp32) elements.
 int check_tensor(const char* who, const char* name, const void* ptr, const AttnStrides& s, int dtype, bool vec) {
   ODY_REQUIRE(ptr != nullptr, ODY_ERR_NULL, "%s: %s is NULL", who, name);
   if (vec) {
@@ -47,7 +46,7 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
   p.causal = causal ? 1 : 0; p.off = Lk - Lq;
   p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
   p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
-  const bool vec = (dtype == ODY_BF16);
+  const bool vec = true;
   if ((rc = check_tensor("ody_attn_fwd", "q", q, p.sq, dtype, vec))) return rc;
   if ((rc = check_tensor("ody_attn_fwd", "k", k, p.sk, dtype, vec))) return rc;
   if ((rc = check_tensor("ody_attn_fwd", "v", v, p.sv, dtype, vec))) return rc;
@@ -65,7 +64,7 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
     return ody_launch_attn_fwd_w8(p, workspace, st);
   }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
-  return ody_launch_attn_fwd_simt(p, D, dtype, st);
+  return ody_launch_attn_fwd_f32(p, D, st);
 }
 
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
@@ -109,13 +108,13 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
   p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
   p.sdo = {sdo_b, sdo_l, sdo_h}; p.sdq = {sdq_b, sdq_l, sdq_h}; p.sdk = {sdk_b, sdk_l, sdk_h};
   p.sdv = {sdv_b, sdv_l, sdv_h};
-  const bool vec = (dtype == ODY_BF16);
+  const bool vec = true;
   const char* who = "ody_attn_bwd";
   if ((rc = check_tensor(who, "q", q, p.sq, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "k", k, p.sk, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "out", out, p.so, dtype, true))) return rc;    // delta pre-pass is vectorised
-  if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, true))) return rc;
+  if ((rc = check_tensor(who, "out", out, p.so, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dq", dq, p.sdq, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dk", dk, p.sdk, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dv", dv, p.sdv, dtype, vec))) return rc;
@@ -133,5 +132,5 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
   if (dtype == ODY_BF16 && D == 128)
     return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
   if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
-  return ody_launch_attn_bwd_simt(p, D, dtype, st);
+  return ody_launch_attn_bwd_f32(p, D, st);
 }

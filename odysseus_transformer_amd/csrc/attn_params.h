@@ -1,4 +1,4 @@
-// Argument block shared by the attention kernels (forward, backward, SIMT fp32).
+// Argument block shared by the attention kernels (forward, backward, bf16 and fp32).
 #pragma once
 #include "ody_common.h"
 
@@ -57,6 +57,7 @@ int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int 
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st);
-int ody_launch_attn_fwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);
-int ody_launch_attn_bwd_simt(const AttnParams& p, int D, int dtype, hipStream_t st);
+// fp32 on the fp32 matrix cores
+int ody_launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t st);
+int ody_launch_attn_bwd_f32(const AttnParams& p, int D, hipStream_t st);
 int ody_launch_attn_delta(const AttnParams& p, int D, int dtype, hipStream_t st);
