@@ -11,8 +11,8 @@
 // C^T = op(B)^T . op(A)^T so that a lane ends up with 4 consecutive N per
 // register quad and writes 8-byte pieces of C rows.
 //
-// fp32: 64 x 64 tiles on the vector ALUs (the fp32 configuration is small and
-// its 1e-4 tolerance rules out bf16 inputs).
+// fp32 (its 1e-4 tolerance rules out bf16 inputs): v_mfma_f32_32x32x2_f32 on
+// 64 x 64 or 128 x 128 workgroup tiles, any shape and alignment.
 #include <type_traits>
 #include "ody_common.h"
 
@@ -554,58 +554,192 @@ int gemm_bf16(int op, const bf16* a, const bf16* b, bf16* c, const bf16* bias, i
   return dispatch_bf16<false, false>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, workspace, workspace_bytes, st);
 }
 
-// ------------------------------------------------------------------ fp32 SIMT
-// A(m, k) = A[m * sam + k * sak], B(k, n) = B[k * sbk + n * sbn]
+// ------------------------------------------------------------------ fp32 MFMA
+constexpr int FK = 32;  // K-slab of the fp32 kernel
+
+__device__ __forceinline__ f32x16 mfma_f32(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// One operand slab (BT rows x FK of K) on its way from global memory to LDS and out again as
+// MFMA fragments.  KC = true: memory is (rows, K) row-major, LDS [BT][FK + 4], a fragment is one
+// 16-byte read.  KC = false: memory is (K, rows) row-major, LDS [FK][BT + 8], a fragment is four
+// 4-byte reads.  Either way k-step 4 j + t of lane half g multiplies K index 8 j + 4 g + t, so
+// both operands of a product agree, and both pitches keep the reads conflict-free.
+template <int BT, bool KC>
+struct F32Tile {
+  static constexpr int PITCH = KC ? FK + 4 : BT + 8;
+  static constexpr int ELEMS = (KC ? BT : FK) * PITCH;
+  static constexpr int CHUNKS = BT * FK / 4 / 256;  // 16-byte pieces per thread
+  f32x4 r[CHUNKS];
+
+  static __device__ __forceinline__ void coord(int c, int& rr, int& kk) {
+    if (KC) { rr = c / (FK / 4); kk = (c % (FK / 4)) * 4; }
+    else { kk = c / (BT / 4); rr = (c % (BT / 4)) * 4; }
+  }
+  // row0: first row (M or N index) of the tile; k0: first K index; out-of-range elements read as 0
+  template <bool VEC>
+  __device__ __forceinline__ void gload(const float* base, int64_t ld, int row0, int k0, int nrows, int K, int tid) {
+#pragma unroll
+    for (int j = 0; j < CHUNKS; j++) {
+      int rr, kk;
+      coord(tid + 256 * j, rr, kk);
+      const int row = row0 + rr, k = k0 + kk;
+      const float* src = KC ? base + (int64_t)row * ld + k : base + (int64_t)k * ld + row;
+      if (VEC) {
+        r[j] = (row < nrows && k < K) ? *reinterpret_cast<const f32x4*>(src) : f32x4{0.f, 0.f, 0.f, 0.f};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const bool ok = KC ? (row < nrows && k + e < K) : (row + e < nrows && k < K);
+          r[j][e] = ok ? src[e] : 0.f;
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void put(float* lds, int tid) const {
+#pragma unroll
+    for (int j = 0; j < CHUNKS; j++) {
+      int rr, kk;
+      coord(tid + 256 * j, rr, kk);
+      *reinterpret_cast<f32x4*>(lds + (KC ? rr * PITCH + kk : kk * PITCH + rr)) = r[j];
+    }
+  }
+  // k-steps 4 j .. 4 j + 3 of row r0 + i
+  static __device__ __forceinline__ f32x4 frag(const float* lds, int r0, int i, int g, int j) {
+    if (KC) return *reinterpret_cast<const f32x4*>(lds + (r0 + i) * PITCH + 8 * j + 4 * g);
+    f32x4 v;
+#pragma unroll
+    for (int t = 0; t < 4; t++) v[t] = lds[(8 * j + 4 * g + t) * PITCH + r0 + i];
+    return v;
+  }
+};
+
+// v_mfma_f32_32x32x2_f32, 4 wavefronts in a 2 x 2 arrangement, each owning WT x WT result tiles
+// of 32 x 32 (a 64 x 64 or 128 x 128 workgroup tile).  One LDS slab; the next one is fetched into
+// registers while the current one is multiplied.  The product is computed as C^T = op(B)^T op(A)^T,
+// so a lane holds 4 consecutive N per register quad and writes 16-byte pieces of C rows.
+// VEC = false (unaligned pointers or extents that are not multiples of 4) moves single floats.
+template <int WT, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                        float* __restrict__ C, const float* __restrict__ bias, int M,
-                                                       int N, int K, int64_t sam, int64_t sak, int64_t sbk,
-                                                       int64_t sbn, int64_t ldc, int accumulate) {
-  constexpr int T = 64, KB = 16;
-  __shared__ float As[KB][T + 4];
-  __shared__ float Bs[KB][T + 4];
-  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
-  const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
-  float acc[4][4] = {};
-  for (int k0 = 0; k0 < K; k0 += KB) {
-    // 64 x 16 elements per operand, 4 per thread; pick the thread->element map that
-    // walks the unit-stride direction of each operand
-    for (int e = tid; e < T * KB; e += 256) {
-      int mm, kk;
-      if (sak == 1) { kk = e % KB; mm = e / KB; } else { mm = e % T; kk = e / T; }
-      const int gm = m0 + mm, gk = k0 + kk;
-      As[kk][mm] = (gm < M && gk < K) ? A[gm * sam + gk * sak] : 0.f;
-      int nn, kb;
-      if (sbk == 1) { kb = e % KB; nn = e / KB; } else { nn = e % T; kb = e / T; }
-      const int gn = n0 + nn, gk2 = k0 + kb;
-      Bs[kb][nn] = (gn < N && gk2 < K) ? B[gk2 * sbk + gn * sbn] : 0.f;
-    }
+                                                       int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
+                                                       int accumulate, int ntn) {
+  constexpr int BT = 64 * WT;
+  constexpr int NCH = (WT == 1) ? 2 : 1;  // never a single chain of dependent MFMAs
+  using TA = F32Tile<BT, A_KC>;
+  using TB = F32Tile<BT, B_KC>;
+  __shared__ __attribute__((aligned(16))) float As[TA::ELEMS];
+  __shared__ __attribute__((aligned(16))) float Bs[TB::ELEMS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = lane & 31, g = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = (blockIdx.x / ntn) * BT, n0 = (blockIdx.x % ntn) * BT;
+
+  f32x16 acc[WT][WT][NCH];
+#pragma unroll
+  for (int a = 0; a < WT; a++)
+#pragma unroll
+    for (int b = 0; b < WT; b++)
+#pragma unroll
+      for (int c = 0; c < NCH; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[a][b][c][r] = 0.f;
+
+  TA ta;
+  TB tb;
+  ta.template gload<VEC>(A, lda, m0, 0, M, K, tid);
+  tb.template gload<VEC>(B, ldb, n0, 0, N, K, tid);
+  for (int k0 = 0; k0 < K; k0 += FK) {
     __syncthreads();
-#pragma unroll
-    for (int kk = 0; kk < KB; kk++) {
-      float a[4], b[4];
-#pragma unroll
-      for (int u = 0; u < 4; u++) a[u] = As[kk][ty * 4 + u], b[u] = Bs[kk][tx * 4 + u];
-#pragma unroll
-      for (int u = 0; u < 4; u++)
-#pragma unroll
-        for (int v = 0; v < 4; v++) acc[u][v] = fmaf(a[u], b[v], acc[u][v]);
-    }
+    ta.put(As, tid);
+    tb.put(Bs, tid);
     __syncthreads();
+    if (k0 + FK < K) {
+      ta.template gload<VEC>(A, lda, m0, k0 + FK, M, K, tid);
+      tb.template gload<VEC>(B, ldb, n0, k0 + FK, N, K, tid);
+    }
+#pragma unroll
+    for (int j = 0; j < FK / 8; j++) {
+      f32x4 af[WT], bf[WT];
+#pragma unroll
+      for (int a = 0; a < WT; a++) af[a] = TA::frag(As, 32 * (wm * WT + a), i, g, j);
+#pragma unroll
+      for (int b = 0; b < WT; b++) bf[b] = TB::frag(Bs, 32 * (wn * WT + b), i, g, j);
+#pragma unroll
+      for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int a = 0; a < WT; a++)
+#pragma unroll
+          for (int b = 0; b < WT; b++)
+            acc[a][b][t % NCH] = mfma_f32(bf[b][t], af[a][t], acc[a][b][t % NCH]);
+    }
   }
+
+  // register r of lane (i, g) of tile (a, b): row m = 32 (wm WT + a) + i, column n = 32 (wn WT + b) + 8 (r / 4) + 4 g + r % 4
 #pragma unroll
-  for (int u = 0; u < 4; u++) {
-    const int m = m0 + ty * 4 + u;
+  for (int a = 0; a < WT; a++) {
+    const int m = m0 + 32 * (wm * WT + a) + i;
     if (m >= M) continue;
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int n = n0 + tx * 4 + v;
-      if (n >= N) continue;
-      float r = acc[u][v];
-      if (bias) r += bias[n];
-      if (accumulate) r += C[(int64_t)m * ldc + n];
-      C[(int64_t)m * ldc + n] = r;
+    for (int b = 0; b < WT; b++) {
+      f32x16 v = acc[a][b][0];
+      if (NCH == 2) v += acc[a][b][NCH - 1];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int n = n0 + 32 * (wn * WT + b) + 8 * q + 4 * g;
+        float* dst = C + (int64_t)m * ldc + n;
+        if (VEC && n + 3 < N) {
+          f32x4 o{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+          if (bias) o += *reinterpret_cast<const f32x4*>(bias + n);
+          if (accumulate) o += *reinterpret_cast<const f32x4*>(dst);
+          *reinterpret_cast<f32x4*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            if (n + e >= N) continue;
+            float o = v[4 * q + e];
+            if (bias) o += bias[n + e];
+            if (accumulate) o += dst[e];
+            dst[e] = o;
+          }
+        }
+      }
     }
   }
+}
+
+template <int WT, bool A_KC, bool B_KC>
+int launch_f32(const float* a, const float* b, float* c, const float* bias, int M, int N, int K, int64_t lda,
+               int64_t ldb, int64_t ldc, int accumulate, bool vec, hipStream_t st) {
+  constexpr int BT = 64 * WT;
+  const int64_t ntm = (M + BT - 1) / BT, ntn = (N + BT - 1) / BT;
+  ODY_REQUIRE(ntm * ntn < ((int64_t)1 << 31), ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d N=%d too large for one launch", M, N);
+  const dim3 grid((unsigned)(ntm * ntn)), blk(256);
+  if (vec)
+    ODY_LAUNCH("gemm_f32", st, (gemm_f32_kernel<WT, A_KC, B_KC, true>), grid, blk, 0, a, b, c, bias, M, N, K, lda,
+               ldb, ldc, accumulate, (int)ntn);
+  else
+    ODY_LAUNCH("gemm_f32", st, (gemm_f32_kernel<WT, A_KC, B_KC, false>), grid, blk, 0, a, b, c, bias, M, N, K, lda,
+               ldb, ldc, accumulate, (int)ntn);
+  return ody_check_launch("gemm_f32");
+}
+
+template <bool A_KC, bool B_KC>
+int dispatch_f32(const float* a, const float* b, float* c, const float* bias, int M, int N, int K, int64_t lda,
+                 int64_t ldb, int64_t ldc, int accumulate, hipStream_t st) {
+  const bool vec = ody_aligned16(a) && ody_aligned16(b) && ody_aligned16(c) && (!bias || ody_aligned16(bias)) &&
+                   lda % 4 == 0 && ldb % 4 == 0 && ldc % 4 == 0 && M % 4 == 0 && N % 4 == 0 && K % 4 == 0;
+  // 128 x 128 tiles once they fill the chip twice over, 64 x 64 tiles below that
+  const int64_t big = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+  if (big >= 512) return launch_f32<2, A_KC, B_KC>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, vec, st);
+  return launch_f32<1, A_KC, B_KC>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, vec, st);
+}
+
+int gemm_f32(int op, const float* a, const float* b, float* c, const float* bias, int M, int N, int K, int64_t lda,
+             int64_t ldb, int64_t ldc, int accumulate, hipStream_t st) {
+  if (op == ODY_GEMM_NT) return dispatch_f32<true, true>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, st);
+  if (op == ODY_GEMM_NN) return dispatch_f32<true, false>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, st);
+  return dispatch_f32<false, false>(a, b, c, bias, M, N, K, lda, ldb, ldc, accumulate, st);
 }
 
 }  // namespace
@@ -628,16 +762,9 @@ extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const voi
               "ody_gemm: leading dimension smaller than the row length (lda=%lld ldb=%lld ldc=%lld)", (long long)lda,
               (long long)ldb, (long long)ldc);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == ODY_F32) {
-    int64_t sam, sak, sbk, sbn;
-    if (op == ODY_GEMM_TN) { sam = 1; sak = lda; } else { sam = lda; sak = 1; }
-    if (op == ODY_GEMM_NT) { sbk = 1; sbn = ldb; } else { sbk = ldb; sbn = 1; }
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
-    ODY_REQUIRE(grid.y <= 65535, ODY_ERR_BAD_SHAPE, "ody_gemm: M=%d too large for the fp32 path", M);
-    ODY_LAUNCH("gemm_f32", st, gemm_f32_kernel, grid, dim3(256), 0, (const float*)A, (const float*)B, (float*)C,
-                       (const float*)bias, M, N, K, sam, sak, sbk, sbn, ldc, accumulate);
-    return ody_check_launch("gemm_f32");
-  }
+  if (dtype == ODY_F32)
+    return gemm_f32(op, (const float*)A, (const float*)B, (float*)C, (const float*)bias, M, N, K, lda, ldb, ldc,
+                    accumulate, st);
   ODY_REQUIRE(dtype == ODY_BF16, ODY_ERR_UNSUPPORTED, "ody_gemm: dtype %d unknown", dtype);
   // 16-byte vectors along the contiguous direction of every matrix
   ODY_REQUIRE(ody_aligned16(A) && ody_aligned16(B) && ((reinterpret_cast<uintptr_t>(C) & 7u) == 0) &&

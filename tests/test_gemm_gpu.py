@@ -84,6 +84,26 @@ def test_bias_accumulate_and_strides_on_interior_tiles(op, dev):
     assert rel_err(out, ref) <= TOL_BF16
 
 
+@pytest.mark.parametrize("shape", [(77, 53, 41), (130, 66, 33), (5, 3, 1), (259, 131, 100), (2901, 2903, 37)],
+                         ids=lambda s: "M%d_N%d_K%d" % s)
+def test_fp32_any_shape_and_alignment(shape, dev):
+    """fp32 takes extents that are not multiples of 4 and views that start on odd elements."""
+    from odysseus_transformer_amd import ops
+    M, N, K = shape
+    print(f"shape={shape}", flush=True)
+    x = randn((M, K + 3), 21)[:, 1:1 + K]
+    w = randn((N, K), 22, std=0.05)
+    dy = randn((M, N + 1), 23)[:, 1:]
+    b = randn((N,), 24)
+    c0 = randn((M, N), 25)
+    xg, wg, dyg = randn((M, K + 3), 21).to(dev)[:, 1:1 + K], w.to(dev), randn((M, N + 1), 23).to(dev)[:, 1:]
+    out = c0.to(dev).clone()
+    ops.gemm(ops.GEMM_NT, xg, wg, bias=b.to(dev), out=out, accumulate=True)
+    assert rel_err(out, x @ w.T + b + c0) <= TOL_F32, "fwd"
+    assert rel_err(ops.gemm(ops.GEMM_NN, dyg, wg), dy @ w) <= TOL_F32, "dgrad"
+    assert rel_err(ops.gemm(ops.GEMM_TN, dyg, xg), dy.T @ x) <= TOL_F32, "wgrad"
+
+
 def test_linearity_at_full_size(dev):
     """Size-independent property at a rank-shard shape: X (W1 + W2)^T == X W1^T + X W2^T
     up to bf16 rounding, and the wgrad of a row-permuted batch is unchanged."""
