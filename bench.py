@@ -30,6 +30,7 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E, published
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32 MFMA, published
 
 # the rank shard the metric is quoted on
 L, H, HKV, D = 32768, 4, 4, 128
@@ -206,6 +207,7 @@ def main():
     out["mfma_sustained"] = mfma_sustained(_lib, dev)
     if not a.no_layer:
         out["layer"] = layer_share(ops, rn, dev, sec)
+        out["fp32"] = fp32_configuration(_lib, ops, dev)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
@@ -262,6 +264,52 @@ def layer_share(ops, rn, dev, attn_sec):
     res["mlp_half_tokens_per_s"] = round(T_MLP / t_mlp_half, 1)
     # one rank advances its 4096-token shard of the 32768-token layer in attn_half + mlp_half
     res["layer_tokens_per_s_per_gpu"] = round(T_MLP / (t_attn_half + t_mlp_half), 1)
+    return res
+
+
+def fp32_configuration(_lib, ops, dev):
+    """The fp32 parity configuration on the GPU (d=512, 8 heads x 64, i=1376, L=2048: one decoder layer forward +
+    backward), and the fp32 kernels at a size that fills the chip, against the 157.3 TFLOP/s fp32 matrix peak."""
+    import types
+    import torch
+    from odysseus_transformer_amd.decoder.odysseus import OdysseusDecoderLayer
+    res = {}
+    Lc, d, Hc, Dc, ic = 2048, 512, 8, 64, 1376
+    cfg = types.SimpleNamespace(hidden_size=d, num_attention_heads=Hc, num_key_value_heads=Hc, head_dim=Dc,
+                                intermediate_size=ic, hidden_act="silu", attention_dropout=0.0, rms_norm_eps=1e-6,
+                                rope_theta=10000.0, max_position_embeddings=1 << 20, pretraining_tp=1,
+                                num_hidden_layers=1)
+    layer = OdysseusDecoderLayer(cfg).to(dev)
+    g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        for w in layer.parameters():
+            if w.dim() > 1:
+                w.copy_((torch.randn(w.shape, generator=g) * 0.02).to(dev))
+    x = torch.randn((1, Lc, d), generator=g).to(dev).requires_grad_(True)
+    dy = torch.randn((1, Lc, d), generator=g).to(dev)
+    pos = torch.arange(Lc, device=dev)[None]
+
+    def layer_step():
+        layer(x, position_ids=pos).backward(dy)
+
+    res["layer_L2048_d512_ms"] = round(time_gpu(layer_step, 10, 3) * 1e3, 3)
+    res["layer_L2048_d512_tokens_per_s"] = round(Lc / (res["layer_L2048_d512_ms"] * 1e-3), 1)
+
+    La, Ha = 16384, 8
+    q, k, v, do = (torch.randn((1, La, Ha, Dc), generator=g).to(dev) for _ in range(4))
+    o, lse = ops.attn_fwd(q, k, v, causal=True)
+    f_fwd, f_bwd = attn_flops(La, La, Ha, Dc)
+    tf = time_gpu(lambda: ops.attn_fwd(q, k, v, causal=True), 3, 1)
+    tb = time_gpu(lambda: ops.attn_bwd(q, k, v, o, lse, do, causal=True), 3, 1)
+    res["attention_L16384_8x64"] = {"fwd_ms": round(tf * 1e3, 3), "bwd_ms": round(tb * 1e3, 3),
+                                    "fwd_tflops": round(f_fwd / tf / 1e12, 1), "bwd_tflops": round(f_bwd / tb / 1e12, 1),
+                                    "frac_of_fp32_peak": round((f_fwd + f_bwd) / (tf + tb) / 1e12 / PEAK_FP32_TFLOPS, 3)}
+    del q, k, v, do, o, lse
+    M = N = K = 4096
+    a, b, c = (torch.randn((M, K), generator=g).to(dev) for _ in range(3))
+    ts = [time_gpu(lambda op=op: ops.gemm(op, a, b), 3, 1) for op in (ops.GEMM_NT, ops.GEMM_NN, ops.GEMM_TN)]
+    res["gemm_4096x4096x4096"] = {"tflops_nt_nn_tn": [round(2.0 * M * N * K / t / 1e12, 1) for t in ts],
+                                  "frac_of_fp32_peak": round(2.0 * M * N * K / max(ts) / 1e12 / PEAK_FP32_TFLOPS, 3)}
     return res
 
 

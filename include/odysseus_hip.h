@@ -12,8 +12,8 @@
  *     allocates, frees or keeps a pointer after the call returns;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*); no entry
  *     point synchronises the device;
- *   - `dtype` is ODY_BF16 (bf16 storage, fp32 accumulation, MFMA) or ODY_F32
- *     (fp32 storage and arithmetic);
+ *   - `dtype` is ODY_BF16 (bf16 storage, fp32 accumulation, bf16 MFMA) or ODY_F32
+ *     (fp32 storage and arithmetic, fp32 MFMA);
  *   - strides are in ELEMENTS; the innermost (head_dim / feature) stride is 1;
  *   - return value: 0 on success, a negative ody_status otherwise;
  *     ody_last_error() returns a thread-local message for the last failure.
@@ -73,7 +73,8 @@ int ody_mfma_probe(const void* operands, float* sink, int blocks, int iters, voi
  * lse (B, Hq, Lq) fp32 contiguous, natural-log units; -inf for a query row that
  *                      sees no key (its out row is 0).
  * GQA: q head h reads kv head h / (Hq / Hkv).  causal != 0 masks key j for
- * query i when j > i + (Lk - Lq).  D in {64, 128}.
+ * query i when j > i + (Lk - Lq).  D in {64, 128}.  Every tensor: 16-byte aligned
+ * pointer, strides that are multiples of 16 bytes (8 bf16 / 4 fp32 elements).
  * workspace: ody_attn_fwd_workspace_bytes(...) bytes, 256-byte aligned (the bf16
  * head_dim-128 kernel keeps a transposed copy of V and one int per 256-query block
  * there; 0 bytes = may be NULL).
@@ -136,6 +137,8 @@ int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk, const flo
  *                                                           utils/linear_zero3.py:74
  * bias (N) of `dtype` or NULL is added to every row (utils/linear_tpsp.py:175-176).
  * If accumulate != 0, C += result (C read in `dtype`, added in fp32).
+ * bf16: A and B 16-byte aligned with lda, ldb, N and their contiguous extents multiples of 8, C and
+ * bias 8-byte aligned with ldc a multiple of 4.  fp32: any shape and alignment.
  * workspace (optional, 16-byte aligned): with ody_gemm_workspace_bytes(...) > 0 bytes of it a product
  * with a long K and few output tiles (a weight gradient) is computed over several ranges of K at once
  * and summed in fp32; without it (NULL / too small) the same result comes from one pass over K.
