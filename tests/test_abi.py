@@ -42,6 +42,9 @@ def test_validation_returns_codes_without_a_gpu():
     with pytest.raises(_lib.OdysseusHipError) as e:
         _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 2, 2, 96, *([128] * 12), 1.0, 1, 0, 0, 0, 0)
     assert e.value.code == -2
+    with pytest.raises(_lib.OdysseusHipError) as e:     # fp32 row stride of 130 elements: rows not 16-byte aligned
+        _lib.call("ody_attn_fwd", 16, 16, 16, 16, 16, 1, 8, 8, 2, 2, 128, 128, 130, *([128] * 10), 1.0, 1, 1, 0, 0, 0)
+    assert e.value.code == -3
     with pytest.raises(_lib.OdysseusHipError) as e:
         _lib.call("ody_rmsnorm_fwd", 16, 16, 16, 0, 4, 7, 1e-6, 0, 0)
     assert e.value.code == -2

@@ -170,3 +170,26 @@ def test_attention_random_shapes(case, dev):
     assert rel_err(dq, dq_ref, floor) <= TOL_BF16, "dq"
     assert rel_err(dk, dk_ref, floor) <= TOL_BF16, "dk"
     assert rel_err(dv, dv_ref) <= TOL_BF16, "dv"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("case", _random_cases(10, 77), ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d" % c)
+def test_attention_random_shapes_fp32(case, D, dev):
+    """The fp32 kernels on ragged lengths around their 32- and 128-row tiles, key offsets and groups."""
+    from odysseus_transformer_amd import ops
+    B, Lq, Lk, Hq, Hkv, causal = case
+    print(f"case={case} D={D}", flush=True)
+    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, D, torch.float32, seed=Lq * 5 + Lk + D)
+    o_ref, lse_ref = oracle.attention_fwd(q, k, v, causal=causal)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q, k, v, o_ref, lse_ref, do, causal=causal)
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
+    dq0 = randn((B, Lq, Hq, D), 99).to(dev)
+    dq = dq0.clone()
+    _, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=dq, accumulate_dq=True)
+    floor = 1.0 if Lk == 1 else 1e-3
+    assert rel_err(o, o_ref) <= TOL_F32
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    assert rel_err(dq - dq0, dq_ref, floor) <= 4 * TOL_F32, "dq"      # the difference of two rounded sums
+    assert rel_err(dk, dk_ref, floor) <= TOL_F32, "dk"
+    assert rel_err(dv, dv_ref) <= TOL_F32, "dv"
