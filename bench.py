@@ -206,14 +206,14 @@ def main():
     # context for the roofline: the rate a register-only MFMA loop sustains on this box
     out["mfma_sustained"] = mfma_sustained(_lib, dev)
     if not a.no_layer:
-        out["layer"] = layer_share(ops, rn, dev, sec)
+        out["layer"] = layer_share(_lib, ops, rn, dev, sec)
         out["fp32"] = fp32_configuration(_lib, ops, dev)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 
 
-def layer_share(ops, rn, dev, attn_sec):
+def layer_share(_lib, ops, rn, dev, attn_sec):
     """Times the rest of the rank's share of the layer: the TP-split QKV / O linears over
     the gathered 32768 tokens, RoPE, and the sequence shard's RMSNorm + SwiGLU MLP over
     4096 tokens, each forward and backward (fwd, dgrad, wgrad)."""
@@ -233,9 +233,20 @@ def layer_share(ops, rn, dev, attn_sec):
         return tf + td + tw
 
     def membound(tag, fn, nbytes):
+        # wall clock per call (what the layer total uses; for kernels this short it includes the host's
+        # launch cost) and the kernels' own duration from HIP events on the launch stream (the HBM rate)
         t = time_gpu(fn, 10, 3)
-        res[tag] = {"ms": round(t * 1e3, 4), "algorithmic_GBs": round(nbytes / t / 1e9, 1),
-                    "frac_of_hbm_peak": round(nbytes / t / 1e9 / PEAK_HBM_GBS, 3)}
+        _lib.profile_enable(True)
+        _lib.profile_collect()
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        prof = _lib.profile_collect()
+        _lib.profile_enable(False)
+        tk = sum(total_ms for (_, total_ms, _) in prof.values()) / 10 * 1e-3
+        res[tag] = {"ms": round(t * 1e3, 4), "kernel_ms": round(tk * 1e3, 4), "kernels": sorted(prof),
+                    "algorithmic_GBs": round(nbytes / tk / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / tk / 1e9 / PEAK_HBM_GBS, 3)}
         return t
 
     t_attn_half = attn_sec
