@@ -35,6 +35,14 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def _same(ref: torch.Tensor, ref_name: str, **others: torch.Tensor) -> None:
+    """Every tensor has the dtype, device and shape of `ref` (the kernels read raw pointers)."""
+    for name, t in others.items():
+        if t.dtype != ref.dtype or t.device != ref.device or t.shape != ref.shape:
+            raise ValueError(f"{name} must match {ref_name} ({tuple(ref.shape)}, {ref.dtype}, {ref.device}); "
+                             f"got {tuple(t.shape)}, {t.dtype}, {t.device}")
+
+
 def _blhd(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
     if t.dim() != 4:
         raise ValueError(f"{name} must be (B, L, H, D), got {tuple(t.shape)}")
@@ -49,10 +57,12 @@ def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=No
     _need_gpu(q, k, v)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
-    if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D:
-        raise ValueError(f"k {tuple(k.shape)} / v {tuple(v.shape)} do not match q {tuple(q.shape)}")
+    if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"k {tuple(k.shape)} {k.dtype} / v {tuple(v.shape)} {v.dtype} do not match "
+                         f"q {tuple(q.shape)} {q.dtype}")
     if out is None:
         out = torch.empty((B, Lq, Hq, D), dtype=q.dtype, device=q.device)
+    _same(q, "q", out=out)
     lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     ws_bytes = _lib.load().ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
@@ -75,6 +85,10 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
         dq = torch.empty_like(q)
     dk = torch.empty_like(k) if dk is None else dk
     dv = torch.empty_like(v) if dv is None else dv
+    _same(q, "q", out=out, dout=dout, dq=dq)
+    _same(k, "k", v=v, dk=dk, dv=dv)
+    if k.dtype != q.dtype or k.shape[0] != B or k.shape[3] != D or tuple(lse.shape) != (B, Hq, Lq):
+        raise ValueError(f"k {tuple(k.shape)} {k.dtype} / lse {tuple(lse.shape)} do not match q {tuple(q.shape)} {q.dtype}")
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     lib = _lib.load()
     ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
@@ -128,6 +142,10 @@ def gemm(op: int, a, b, bias=None, out=None, accumulate: bool = False):
         if accumulate:
             raise ValueError("accumulate needs an existing out")
         out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    if tuple(out.shape) != (M, N) or out.dtype != a.dtype:
+        raise ValueError(f"out must be ({M}, {N}) {a.dtype}, got {tuple(out.shape)} {out.dtype}")
+    if bias is not None and (tuple(bias.shape) != (N,) or bias.dtype != a.dtype or not bias.is_contiguous()):
+        raise ValueError(f"bias must be a contiguous ({N},) {a.dtype} tensor, got {tuple(bias.shape)} {bias.dtype}")
     ws_bytes = _lib.load().ody_gemm_workspace_bytes(op, M, N, K, _dt(a))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     _lib.call("ody_gemm", op, a.data_ptr(), b.data_ptr(), out.data_ptr(), 0 if bias is None else bias.data_ptr(),
