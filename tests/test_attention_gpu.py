@@ -20,6 +20,8 @@ CASES = [
     (1, 192, 320, 4, 2, 128, True),      # causal with key offset
     (1, 1, 1, 1, 1, 128, True),          # single token
     (1, 1024, 1024, 4, 1, 128, True),
+    (1, 300, 100, 4, 2, 128, True),      # fewer keys than queries: the first 200 queries see no key
+    (2, 200, 72, 8, 8, 64, True),        # the same at head_dim 64
 ]
 
 
