@@ -141,3 +141,49 @@ def test_patched_hf_llama_runs_and_matches_oracle(dev):
     logits.float().square().mean().backward()
     assert model.model.layers[0].self_attn.qkv_proj.weight.grad is not None
     assert torch.isfinite(model.model.embed_tokens.weight.grad).all()
+
+
+@pytest.mark.parametrize("case", [LAYER_CASES[0], LAYER_CASES[2]], ids=lambda c: c[0])
+def test_layer_step_replayed_from_a_hip_graph(case, dev):
+    """No entry point allocates, synchronises or clears memory with a memset, so a whole layer step
+    (forward + backward) can be captured into a HIP graph.  Every replay -- with eager work and
+    synchronisations in between -- must reproduce the eager result bit for bit."""
+    from odysseus_transformer_amd.decoder.odysseus import OdysseusDecoderLayer
+    name, L, d, H, Hkv, D, i, dtype = case
+    print(f"graph case {name}", flush=True)
+    layer = _load(OdysseusDecoderLayer(_config(d, H, Hkv, D, i)).to(dtype), _params(d, H, Hkv, D, i, dtype), dev)
+    params = list(layer.parameters())
+    x = randn((1, L, d), 31, dtype=dtype).to(dev).requires_grad_(True)
+    dy = randn((1, L, d), 32, dtype=dtype).to(dev)
+    pos = torch.arange(L, device=dev)[None]
+
+    def step():
+        for t in params + [x]:
+            t.grad = None
+        y = layer(x, position_ids=pos)
+        y.backward(dy)
+        return y
+
+    side = torch.cuda.Stream()                      # warm-up off the default stream, as graph capture requires
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            y = step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = [y.detach().clone(), x.grad.clone()] + [t.grad.clone() for t in params]
+    del y                                           # drops the warm-up's autograd graph
+
+    for t in params + [x]:
+        t.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_g = layer(x, position_ids=pos)
+        y_g.backward(dy)
+    captured = [y_g.detach(), x.grad] + [t.grad for t in params]
+    for replay in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), f"replay {replay} differs from the eager step"
+        float(torch.randn(4096, device=dev).square().sum())   # eager work and a synchronisation between replays
