@@ -186,6 +186,17 @@ def main():
     traffic = measured_traffic().get(dom)
     value = (f_fwd + f_bwd) / sec / 1e12
 
+    info = _lib.device_info()
+    device = {"name": prop.name, "cus": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0,
+              "lds_bytes_per_cu": info["lds_bytes_per_cu"],
+              # 4 SIMDs x one 32x32x16 bf16 MFMA (32768 FLOP) per 32 cycles = 4096 FLOP per clock per CU
+              "bf16_peak_from_cus_and_clock_tflops": round(info["compute_units"] * info["clock_khz"] * 1e3 * 4096 / 1e12, 1)}
+    # kernels of the forward: the V image (one of the step's four image launches), the main kernel and
+    # its follow-up over flagged query blocks; everything else belongs to the backward
+    fwd_ms = (prof["attn_fwd_w8"][1] + prof.get("attn_fwd_mfma", (0, 0.0, 0))[1] +
+              prof.get("attn_images", (0, 0.0, 0))[1] / 4) / a.steps
+    bwd_ms = sum(t for n, (_, t, _) in prof.items()) / a.steps - fwd_ms
+
     out = {
         "metric": "attention fwd+bwd TFLOP/s (% bf16 MFMA peak) + decoder-layer tokens/s, 1 GPU",
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -193,10 +204,12 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "causal attention fwd+bwd, Llama-2-7B rank shard at N=8: 4 heads x 128, L=32768, "
                                "batch 1 (attention part of the 32768-token bf16 configuration)",
-                   "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd},
+                   "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd,
+                   "seeds": {"qkv": 2001, "dout": 2002}},
+        "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
+        "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 1), "bwd_tflops": round(f_bwd / (bwd_ms * 1e-3) / 1e12, 1),
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
-        "device": {"name": prop.name, "cus": prop.multi_processor_count,
-                   "clock_mhz": getattr(prop, "clock_rate", 0) / 1000.0},
+        "device": device,
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 1), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
                      "avg_ms": round(dom_avg, 4), "algorithmic_flops_per_launch": algo[dom]},

@@ -44,6 +44,13 @@ enum ody_status {
 const char* ody_last_error(void);
 int ody_version(void);
 
+/* The current device as the kernels see it (no counterpart in the reference): compute units, the
+ * engine clock in kHz and the LDS bytes of one compute unit.  Any pointer may be NULL.  The bf16
+ * matrix peak follows as compute_units * clock * 4096 FLOP per clock (4 SIMDs, one 32x32x16 MFMA
+ * per 32 cycles each).
+ */
+int ody_device_info(int* compute_units, int* clock_khz, int* lds_bytes_per_cu);
+
 /* Per-kernel timer (no counterpart in the reference, whose only clock is time.time()
  * around whole steps, train.py:185-229).  While enabled, every kernel launch of the
  * library is bracketed by a pair of HIP events on its launch stream.

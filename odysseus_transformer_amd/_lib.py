@@ -20,6 +20,7 @@ _i, _i64, _f, _p, _sz = C.c_int, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
 SIGNATURES = {
     "ody_last_error": (C.c_char_p, []),
     "ody_version": (_i, []),
+    "ody_device_info": (_i, [_p, _p, _p]),
     "ody_profile_enable": (_i, [_i]),
     "ody_profile_collect": (_i, [C.c_char_p, _sz]),
     "ody_mfma_probe": (_i, [_p, _p, _i, _i, _p]),
@@ -73,6 +74,13 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise OdysseusHipError(name, rc, lib.ody_last_error().decode("utf-8", "replace"))
+
+
+def device_info() -> dict:
+    """Compute units, engine clock (kHz) and LDS bytes per compute unit of the current device."""
+    cu, khz, lds = C.c_int(0), C.c_int(0), C.c_int(0)
+    call("ody_device_info", C.addressof(cu), C.addressof(khz), C.addressof(lds))
+    return {"compute_units": cu.value, "clock_khz": khz.value, "lds_bytes_per_cu": lds.value}
 
 
 def profile_enable(on: bool) -> None:

@@ -51,6 +51,26 @@ OdyKernelScope::~OdyKernelScope() {
 extern "C" const char* ody_last_error(void) { return g_err; }
 extern "C" int ody_version(void) { return 1; }
 
+extern "C" int ody_device_info(int* compute_units, int* clock_khz, int* lds_bytes_per_cu) {
+  int dev = 0, v = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    ody_set_error("ody_device_info: no current HIP device");
+    return ODY_ERR_LAUNCH;
+  }
+  const hipDeviceAttribute_t what[3] = {hipDeviceAttributeMultiprocessorCount, hipDeviceAttributeClockRate,
+                                        hipDeviceAttributeMaxSharedMemoryPerMultiprocessor};
+  int* const where[3] = {compute_units, clock_khz, lds_bytes_per_cu};
+  for (int k = 0; k < 3; k++) {
+    if (!where[k]) continue;
+    if (hipDeviceGetAttribute(&v, what[k], dev) != hipSuccess) {
+      ody_set_error("ody_device_info: hipDeviceGetAttribute failed");
+      return ODY_ERR_LAUNCH;
+    }
+    *where[k] = v;
+  }
+  return ODY_OK;
+}
+
 extern "C" int ody_profile_enable(int on) {
   std::lock_guard<std::mutex> lk(g_mu);
   g_profile = on != 0;
