@@ -9,7 +9,7 @@ hold for any input (sum_j dV_j == sum_i dO_i, sum_j dK_j == 0) cover the rest.
 import pytest
 import torch
 
-from conftest import TOL_BF16, TOL_LSE, randn, rel_err
+from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
 import odysseus_oracle as oracle
 from sampled import edge_samples, sampled_checks
 
@@ -54,6 +54,19 @@ def test_long_sequences_sampled(L, Hq, Hkv, dev):
     o, lse, dq, dk, dv = run_attention(q, k, v, do, dev)
     sampled_checks(q[0], k[0], v[0], do[0], o[0], lse[0], dq[0], dk[0], dv[0], True,
                    edge_samples(L, 16, 1), edge_samples(L, 8, 2))
+
+
+def test_fp32_long_sequence_sampled(dev):
+    """The fp32 kernels at a length that fills the chip: 8 query heads x 64 over 2 kv heads, L = 16384."""
+    L, Hq, Hkv, D = 16384, 8, 2, 64
+    print(f"fp32 attention L={L} Hq={Hq} Hkv={Hkv}, sampled fp64 parity", flush=True)
+    q = randn((1, L, Hq, D), 3100)
+    k = randn((1, L, Hkv, D), 3101)
+    v = randn((1, L, Hkv, D), 3102)
+    do = randn((1, L, Hq, D), 3103)
+    o, lse, dq, dk, dv = run_attention(q, k, v, do, dev)
+    sampled_checks(q[0], k[0], v[0], do[0], o[0], lse[0], dq[0], dk[0], dv[0], True,
+                   edge_samples(L, 16, 3), edge_samples(L, 8, 4), tol=TOL_F32)
 
 
 def test_cfg5_ring_of_eight_blocks_sampled(dev):
