@@ -119,6 +119,10 @@ def main():
                     help="also run one plain device copy of the packed qkv buffer (100 MiB read + 100 MiB "
                          "written): the known-size kernel that calibrates the HBM byte counters of a "
                          "rocprofv3 --pmc run of this script")
+    ap.add_argument("--power", action="store_true",
+                    help="also read package power and engine clock from rocm-smi while the step, a GEMM, the MFMA "
+                         "probe and a plain copy each run in a loop for a few seconds (slow: rocm-smi takes seconds "
+                         "per reading)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU's share of the layer on ONE GPU; collectives and multi-GPU runs are "
@@ -221,6 +225,8 @@ def main():
     if not a.no_layer:
         out["layer"] = layer_share(_lib, ops, rn, dev, sec)
         out["fp32"] = fp32_configuration(_lib, ops, dev)
+    if a.power:
+        out["power"] = power_under_load(_lib, ops, dev, step)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
@@ -289,6 +295,50 @@ def layer_share(_lib, ops, rn, dev, attn_sec):
     # one rank advances its 4096-token shard of the 32768-token layer in attn_half + mlp_half
     res["layer_tokens_per_s_per_gpu"] = round(T_MLP / (t_attn_half + t_mlp_half), 1)
     return res
+
+
+def power_under_load(_lib, ops, dev, attention_step):
+    """Package power (W) and engine clock (MHz) as rocm-smi reports them while one workload at a time keeps
+    the queue full: the matrix kernels run at the package power limit, and the clock is what gives."""
+    import subprocess
+    import torch
+
+    def reading():
+        txt = subprocess.run(["/opt/rocm/bin/rocm-smi", "-a", "--json"], capture_output=True, text=True).stdout
+        card = json.loads(txt[txt.index("{"):])["card0"]
+        return {"socket_power_w": card.get("current_socket_power (W)"), "sclk": card.get("sclk clock speed:"),
+                "power_limit_w": card.get("Max Graphics Package Power (W)"),
+                "junction_c": card.get("Temperature (Sensor junction) (C)")}
+
+    def under(fn, secs=4.0):
+        fn()
+        torch.cuda.synchronize()
+        t0, got = time.time(), None
+        while time.time() - t0 < secs or got is None:
+            for _ in range(20):
+                fn()
+            if time.time() - t0 > 1.5 and got is None:
+                got = reading()          # taken while 20 launches are still queued
+        torch.cuda.synchronize()
+        return got
+
+    st = torch.cuda.current_stream().cuda_stream
+    rand = torch.randn(1 << 20, device=dev).bfloat16()
+    ones = torch.ones(1 << 20, device=dev).bfloat16()
+    sink = torch.empty(4096 * 256, device=dev)
+    a = torch.randn((8192, 8192), device=dev).bfloat16()
+    b = torch.randn((8192, 8192), device=dev).bfloat16()
+    src = torch.randn(1 << 28, device=dev).bfloat16()
+    dst = torch.empty_like(src)
+    return {
+        "attention_step": under(attention_step),
+        "gemm_nt_8192": under(lambda: ops.gemm(ops.GEMM_NT, a, b)),
+        "mfma_probe_random_operands": under(lambda: _lib.call("ody_mfma_probe", rand.data_ptr(), sink.data_ptr(), 4096,
+                                                              2000, st)),
+        "mfma_probe_constant_operands": under(lambda: _lib.call("ody_mfma_probe", ones.data_ptr(), sink.data_ptr(),
+                                                                4096, 2000, st)),
+        "copy_512MiB": under(lambda: dst.copy_(src)),
+    }
 
 
 def fp32_configuration(_lib, ops, dev):
