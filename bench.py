@@ -103,9 +103,23 @@ def cpu_baseline():
     oracle.attention_bwd(q, k, v, o, lse, do, causal=True)
     dt = time.perf_counter() - t0
     f, b = attn_flops(Ls, Ls, H, D)
+    # the fp32 configuration as a whole on the same cores: one decoder layer forward + backward,
+    # d=512, 8 heads x 64, i=1376, L=2048 (3 warm-up runs, 10 timed)
+    Lc, dc, Hc, Dc, ic = 2048, 512, 8, 64, 1376
+    w = {"ln1": torch.ones(dc), "ln2": torch.ones(dc),
+         "w_qkv": torch.randn(3 * Hc * Dc, dc, generator=g) * 0.02, "w_o": torch.randn(dc, Hc * Dc, generator=g) * 0.02,
+         "w_gate_up": torch.randn(2 * ic, dc, generator=g) * 0.02, "w_down": torch.randn(dc, ic, generator=g) * 0.02}
+    x, dy = torch.randn(1, Lc, dc, generator=g), torch.randn(1, Lc, dc, generator=g)
+    for _ in range(3):
+        oracle.decoder_layer_fwd_bwd(x, w, dy, Hc, Hc, Dc)
+    t0 = time.perf_counter()
+    for _ in range(10):
+        oracle.decoder_layer_fwd_bwd(x, w, dy, Hc, Hc, Dc)
+    layer_ms = (time.perf_counter() - t0) / 10 * 1e3
     return {"value": (f + b) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"causal attention fwd+bwd, {H} heads x {D}, L={Ls} (1/4 of the step's FLOPs), fp32, "
-                      f"{dt:.2f} s wall"}
+                      f"{dt:.2f} s wall",
+            "fp32_layer_L2048_d512_ms": round(layer_ms, 2)}
 
 
 def main():
