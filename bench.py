@@ -236,6 +236,8 @@ def main():
 
     # context for the roofline: the rate a register-only MFMA loop sustains on this box
     out["mfma_sustained"] = mfma_sustained(_lib, dev)
+    # boxes differ by ~10 % in what they sustain at the power limit; this ratio does not
+    out["value_over_mfma_sustained_random"] = round(value / out["mfma_sustained"]["random_operands_tflops"], 3)
     if not a.no_layer:
         out["layer"] = layer_share(_lib, ops, rn, dev, sec)
         out["fp32"] = fp32_configuration(_lib, ops, dev)
