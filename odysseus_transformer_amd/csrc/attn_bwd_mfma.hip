@@ -73,7 +73,7 @@ __device__ __forceinline__ bf16x8 lds_tr_frag(const bf16* tile, int row32, int s
 // dK / dV
 // ---------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
   constexpr int BQ = 64, WK = 32, BN = 4 * WK, P = D + 8, KS = D / 16, DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* Qs = reinterpret_cast<bf16*>(smem_raw);       // [2][BQ][P]
