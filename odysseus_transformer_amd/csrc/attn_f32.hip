@@ -94,6 +94,23 @@ __device__ __forceinline__ void tile_times_frag(const float* tile, int i, int g,
   }
 }
 
+// Two products of that kind at once, interleaved: each is the other's independent chain.
+template <int D>
+__device__ __forceinline__ void tiles_times_frags(const float* ta, const float (&fa)[D / 2], f32x16& ca, const float* tb,
+                                                  const float (&fb)[D / 2], f32x16& cb, int i, int g) {
+  constexpr int LD = D + 4;
+#pragma unroll
+  for (int j = 0; j < D / 8; j++) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(ta + i * LD + 8 * j + 4 * g);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(tb + i * LD + 8 * j + 4 * g);
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      ca = mfma_f32(a[t], fa[4 * j + t], ca);
+      cb = mfma_f32(b[t], fb[4 * j + t], cb);
+    }
+  }
+}
+
 // acc[db] += T^T W for a 32-row LDS tile T (its 32 rows are contracted) and the weights
 // W held in result-register order; D / 32 independent chains.
 template <int D>
@@ -266,13 +283,10 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnPa
     }
     if (n0 >= w_end) continue;
 
-    f32x16 s, s1, dp, dp1;
+    f32x16 s, dp;
 #pragma unroll
-    for (int r = 0; r < 16; r++) s[r] = s1[r] = dp[r] = dp1[r] = 0.f;
-    tile_times_frag<D>(Ks, i, g, qf, s, s1);    // S^T  = K Q^T   (log2 domain)
-    tile_times_frag<D>(Vs, i, g, dof, dp, dp1);  // dP^T = V dO^T
-    s += s1;
-    dp += dp1;
+    for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
+    tiles_times_frags<D>(Ks, qf, s, Vs, dof, dp, i, g);  // S^T = K Q^T (log2 domain), dP^T = V dO^T
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const float pr = (n0 + acc_row(r, g) > lim) ? 0.f : ody_exp2(s[r] - lse2);
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnPa
 // accumulators do not fit the register file together, so dV and dK take a pass each.)
 // ---------------------------------------------------------------------------------------
 template <int D, int WHICH>
-__global__ __launch_bounds__(F_THREADS) void attn_bwd_dkdv_f32_kernel(const AttnParams p) {
+__global__ __launch_bounds__(F_THREADS, (D == 64 || WHICH == 0) ? 2 : 1) void attn_bwd_dkdv_f32_kernel(const AttnParams p) {
   constexpr int LD = D + 4, NDB = D / 32;
   constexpr bool DO_DV = (WHICH != 1), DO_DK = (WHICH != 0);
   __shared__ __attribute__((aligned(16))) float Qs[F_TILE * LD];
@@ -354,18 +368,15 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dkdv_f32_kernel(const Attn
       if (i0 + F_TILE < p.Lq) fetch(i0 + F_TILE);
       if (i0 + F_TILE <= w_begin || wn0 >= p.Lk) continue;  // wavefront-uniform
 
-      f32x16 s, s1;
+      // S = Q K^T (log2 domain): rows = queries, column = this lane's key; dP = dO V^T
+      f32x16 s, dp;
 #pragma unroll
-      for (int r = 0; r < 16; r++) s[r] = s1[r] = 0.f;
-      tile_times_frag<D>(Qs, i, g, kf, s, s1);  // S = Q K^T (log2 domain): rows = queries, column = this lane's key
-      s += s1;
-      f32x16 dp;
+      for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
       if constexpr (DO_DK) {
-        f32x16 dp1;
-#pragma unroll
-        for (int r = 0; r < 16; r++) dp[r] = dp1[r] = 0.f;
-        tile_times_frag<D>(Os, i, g, vf, dp, dp1);  // dP = dO V^T
-        dp += dp1;
+        tiles_times_frags<D>(Qs, kf, s, Os, vf, dp, i, g);
+      } else {
+        tile_times_frag<D>(Qs, i, g, kf, s, dp);
+        s += dp;
       }
       f32x4 lv[4], dl[4];
 #pragma unroll
