@@ -144,7 +144,7 @@ __device__ __forceinline__ void store_rows(float* dst, const f32x16 (&acc)[D / 3
 // forward
 // ---------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(F_THREADS) void attn_fwd_f32_kernel(const AttnParams p) {
+__global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kernel(const AttnParams p) {
   constexpr int LD = D + 4, NDB = D / 32;
   __shared__ __attribute__((aligned(16))) float Ks[F_TILE * LD];
   __shared__ __attribute__((aligned(16))) float Vs[F_TILE * LD];
