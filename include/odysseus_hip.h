@@ -196,6 +196,26 @@ int ody_rope(void* x, const int64_t* position_ids, const float* inv_freq, int B,
              int D, int64_t sx_b, int64_t sx_l, int64_t sx_h, float base, int inverse,
              int dtype, void* stream);
 
+/* ---- cross-entropy over the vocabulary --------------------------------------
+ * flash_attn.losses.cross_entropy.CrossEntropyLoss(inplace_backward=True) as the training loop
+ * uses it (train.py:8,173,212-214): softmax cross-entropy of logits (T, V) (row stride ld,
+ * `dtype`) against labels (T) int64, statistics in fp32.
+ * fwd: lse (T) = log sum_v exp(logits[t, v]); losses (T) = lse[t] - logits[t, labels[t]], and 0
+ *      for a token whose label is ignore_index (or outside [0, V): such a token is skipped, never
+ *      dereferenced).  If reduced != NULL: reduced[0] = mean of the losses over the counted
+ *      tokens, reduced[1] = their number (one block, fixed order: deterministic).
+ * bwd: overwrites logits IN PLACE with d loss / d logits = (softmax - onehot(label)) * g, where
+ *      g = dloss[t] if dloss != NULL (per-token upstream gradient), else grad_loss[0] / reduced[1]
+ *      (mean reduction; grad_loss is a DEVICE scalar, so nothing synchronises).  Rows of skipped
+ *      tokens become 0.
+ * 16-byte accesses are used when logits is 16-byte aligned and ld a multiple of 8 (bf16) / 4 (fp32).
+ */
+int ody_cross_entropy_fwd(const void* logits, const int64_t* labels, float* losses, float* lse, float* reduced,
+                          int T, int V, int64_t ld, int64_t ignore_index, int dtype, void* stream);
+int ody_cross_entropy_bwd(void* logits, const int64_t* labels, const float* lse, const float* reduced,
+                          const float* grad_loss, const float* dloss, int T, int V, int64_t ld,
+                          int64_t ignore_index, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,8 @@ SIGNATURES = {
     "ody_rmsnorm_fwd": (_i, [_p] * 4 + [_i, _i, _f, _i, _p]),
     "ody_rmsnorm_bwd_partials": (_i, [_i]),
     "ody_rmsnorm_bwd": (_i, [_p] * 7 + [_i, _i, _i, _p]),
+    "ody_cross_entropy_fwd": (_i, [_p] * 5 + [_i, _i, _i64, _i64, _i, _p]),
+    "ody_cross_entropy_bwd": (_i, [_p] * 6 + [_i, _i, _i64, _i64, _i, _p]),
     "ody_rope": (_i, [_p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _f, _i, _i, _p]),
 }
 

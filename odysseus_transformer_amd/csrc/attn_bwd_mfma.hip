@@ -341,18 +341,10 @@ template <int D>
 int launch(const AttnParams& p, hipStream_t st) {
   constexpr size_t smem_kv = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16) + 2 * 2 * 64 * sizeof(float);
   constexpr size_t smem_q = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
-      ody_set_error("attn_bwd: hipFuncSetAttribute failed");
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D>), smem_kv, "attn_bwd"))
+    return rc;
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D>), smem_q, "attn_bwd"))
+    return rc;
   dim3 gk(((p.Lk + 127) / 128) * p.Hkv * p.B);
   ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
   int rc = ody_check_launch("attn_bwd_dkdv");

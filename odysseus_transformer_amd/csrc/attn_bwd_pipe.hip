@@ -15,6 +15,7 @@
 //
 // dK/dV kernel -- key-stationary, 32 keys per wavefront (described where it is defined).
 #include <type_traits>
+#include <utility>
 #include "attn_params.h"
 #include "attn_tile.h"
 
@@ -503,19 +504,10 @@ size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem_q = (size_t)3 * (2 * TILE_ELEMS + IMG_ELEMS) * sizeof(bf16);
   constexpr size_t smem_kv = (size_t)2 * KV_STAGE * sizeof(bf16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_q) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_kv) != hipSuccess) {
-      ody_set_error("attn_bwd: hipFuncSetAttribute failed");
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  for (const auto& ks : {std::pair<const void*, size_t>{reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel), smem_q},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false>), smem_kv},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true>), smem_kv}})
+    if (int rc = ody_allow_dynamic_lds(ks.first, ks.second, "attn_bwd")) return rc;
   unsigned char* w = static_cast<unsigned char*>(workspace);
   bf16* kimg = reinterpret_cast<bf16*>(w);
   bf16* qimg = reinterpret_cast<bf16*>(w + align256(ody_attn_images_bytes(p.B, p.Lk, p.Hkv)));

@@ -239,16 +239,8 @@ template <int D, int QT>
 int launch(const AttnParams& p, const int* flags, int flag_block, hipStream_t st) {
   constexpr int BN = 64, BM = 4 * 32 * QT;
   constexpr size_t smem = (size_t)2 * BN * ((D + 8) + (D + 32)) * sizeof(bf16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_mfma_kernel<D, QT>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) {
-      ody_set_error("attn_fwd: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_fwd_mfma_kernel<D, QT>), smem, "attn_fwd"))
+    return rc;
   dim3 grid(((p.Lq + BM - 1) / BM) * p.Hq * p.B);
   ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, p, flags, flag_block);
   return ody_check_launch("attn_fwd_mfma");

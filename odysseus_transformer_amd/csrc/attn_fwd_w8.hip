@@ -195,22 +195,14 @@ size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
 
 int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem = (size_t)3 * FW_STAGE * sizeof(bf16);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_w8_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) {
-      ody_set_error("attn_fwd: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_fwd_w8_kernel), smem, "attn_fwd");
+  if (rc) return rc;
   const int nqb = (p.Lq + FW_BM - 1) / FW_BM;
   const int nflags = p.B * p.Hq * nqb;
   int* flags = static_cast<int*>(workspace);
   bf16* images =
       reinterpret_cast<bf16*>(static_cast<char*>(workspace) + (((size_t)nflags * sizeof(int) + 255) & ~(size_t)255));
-  int rc = ody_launch_attn_images(p.v, p.sv, p.B, p.Lk, p.Hkv, images, flags, nflags, st);
+  rc = ody_launch_attn_images(p.v, p.sv, p.B, p.Lk, p.Hkv, images, flags, nflags, st);
   if (rc) return rc;
   dim3 grid(nqb * p.Hq * p.B);
   ODY_LAUNCH("attn_fwd_w8", st, attn_fwd_w8_kernel, grid, dim3(FW_THREADS), smem, p, images, flags);

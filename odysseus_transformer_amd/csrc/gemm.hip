@@ -464,25 +464,12 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
                 int64_t ldc, int accumulate, float* part, int splits, hipStream_t st) {
   constexpr int TM = 64 * WM, TN = 64 * WN;
   constexpr size_t smem = 2 * sizeof(bf16) * (OperandTile<TM, A_KC>::ELEMS + OperandTile<TN, B_KC>::ELEMS);
-  static bool attr_set = false;
   auto kern = &gemm_bf16_kernel<WM, WN, A_KC, B_KC>;
   auto fast = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC, false>;
   auto fastk = &gemm_bf16_fast_kernel<WM, WN, A_KC, B_KC, true>;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)smem);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute(reinterpret_cast<const void*>(fastk), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)smem);
-    if (e != hipSuccess) {
-      ody_set_error("ody_gemm: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-      return ODY_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  for (const void* f : {reinterpret_cast<const void*>(kern), reinterpret_cast<const void*>(fast),
+                        reinterpret_cast<const void*>(fastk)})
+    if (int rc = ody_allow_dynamic_lds(f, smem, "ody_gemm")) return rc;
   const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
   const char* name = A_KC ? (B_KC ? "gemm_bf16_nt" : "gemm_bf16_nn") : "gemm_bf16_tn";
   // per-thread offsets inside a tile are kept in 32 bits by the fast kernel, and it writes C in 16-byte pieces

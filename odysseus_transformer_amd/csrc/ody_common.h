@@ -24,6 +24,10 @@ void ody_set_error(const char* fmt, ...);
 // Returns ODY_OK or ODY_ERR_LAUNCH after a kernel launch (reads hipGetLastError).
 int ody_check_launch(const char* what);
 
+// Raises a kernel's dynamic-LDS limit to `bytes` on the current device.  Done once per (kernel, device)
+// under a lock, so concurrent first calls from several host threads and several devices are safe.
+int ody_allow_dynamic_lds(const void* kernel, size_t bytes, const char* who);
+
 // Brackets one kernel launch with a pair of HIP events on the launch stream when the
 // timer is enabled (ody_profile_enable); costs one branch otherwise.
 struct OdyKernelScope {

@@ -5,6 +5,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <utility>
 #include <vector>
 #include "ody_common.h"
 
@@ -15,6 +16,7 @@ struct Span { const char* name; hipEvent_t start, stop; };
 std::mutex g_mu;
 bool g_profile = false;
 std::vector<Span> g_spans;
+constexpr size_t kMaxSpans = 1u << 18;   // launches kept between two ody_profile_collect calls
 }  // namespace
 
 void ody_set_error(const char* fmt, ...) {
@@ -33,6 +35,26 @@ int ody_check_launch(const char* what) {
   return ODY_OK;
 }
 
+int ody_allow_dynamic_lds(const void* kernel, size_t bytes, const char* who) {
+  static std::mutex mu;
+  static std::vector<std::pair<const void*, int>> done;   // (kernel, device) pairs already raised
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    ody_set_error("%s: no current HIP device", who);
+    return ODY_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lk(mu);
+  for (const auto& kd : done)
+    if (kd.first == kernel && kd.second == dev) return ODY_OK;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) {
+    ody_set_error("%s: hipFuncSetAttribute(%zu bytes of dynamic LDS) failed: %s", who, bytes, hipGetErrorString(e));
+    return ODY_ERR_LAUNCH;
+  }
+  done.emplace_back(kernel, dev);
+  return ODY_OK;
+}
+
 OdyKernelScope::OdyKernelScope(const char* name, hipStream_t st) : name_(name), st_(st), start_(nullptr) {
   if (!g_profile) return;
   if (hipEventCreate(&start_) != hipSuccess) { start_ = nullptr; return; }
@@ -45,6 +67,11 @@ OdyKernelScope::~OdyKernelScope() {
   if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start_); return; }
   (void)hipEventRecord(stop, st_);
   std::lock_guard<std::mutex> lk(g_mu);
+  if (g_spans.size() >= kMaxSpans) {   // nobody collects: drop the span instead of growing without bound
+    (void)hipEventDestroy(start_);
+    (void)hipEventDestroy(stop);
+    return;
+  }
   g_spans.push_back({name_, start_, stop});
 }
 

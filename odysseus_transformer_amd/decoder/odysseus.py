@@ -251,10 +251,24 @@ def _host_layer_unpacks_two(layer) -> bool:
         return False
 
 
+def _host_builds_no_mask(model) -> None:
+    """The modules apply the causal mask themselves and refuse an explicit one.  With the `eager`
+    attention implementation transformers hands every layer a dense causal mask; declaring
+    flash_attention_2 (what the reference's train.py:72,84 asks for) makes the host pass None
+    unless the batch is padded."""
+    cfg = getattr(model, "config", None)
+    if cfg is not None and getattr(cfg, "_attn_implementation", None) not in (None, "flash_attention_2"):
+        try:
+            cfg._attn_implementation = "flash_attention_2"
+        except Exception:   # a host that validates the assignment: the mask check in forward() still guards
+            pass
+
+
 def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True):
     """Swaps every layer's attention (and, by default, MLP) for the Odysseus modules
     (decoder/odysseus.py:298-309).  As in the reference the new modules are freshly
     initialised: pretrained attention / MLP weights are not carried over."""
+    _host_builds_no_mask(model)
     for i in range(model.config.num_hidden_layers):
         layer = model.model.layers[i]
         new_module = LlamaFlashAttention2TPSP(model.config, i).to(model.dtype)

@@ -35,6 +35,23 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def scratch(nbytes: int, name: str, device) -> torch.Tensor:
+    """Kernel scratch of `nbytes` bytes.  When the process-wide arena is set up for this device
+    (utils.globals._set_global_memory_buffer, as the reference's train.py:62 does), the bytes come
+    from its grow-only buffer `name` -- the use the reference makes of it for its gathered
+    activations and weights (utils/linear_tpsp.py:159-165, utils/linear_zero3.py:38-40) -- so that
+    steady-state steps allocate no scratch at all.  Buffers of one name alias each other: the
+    kernels of one stream run in order, which is what makes the reuse safe; work on several
+    streams at once needs the arena off.  Without an arena: a fresh torch allocation."""
+    from .utils import globals as _globals
+    arena = _globals._Arena.instance
+    if arena is not None and nbytes > 0:
+        adev = torch.device(arena.dev)
+        if adev.type == device.type and (adev.index is None or adev.index == device.index):
+            return arena.get_tensor((nbytes,), torch.uint8, name)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def _same(ref: torch.Tensor, ref_name: str, **others: torch.Tensor) -> None:
     """Every tensor has the dtype, device and shape of `ref` (the kernels read raw pointers)."""
     for name, t in others.items():
@@ -66,7 +83,7 @@ def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=No
     lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     ws_bytes = _lib.load().ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    ws = scratch(ws_bytes, "attn_fwd_workspace", q.device) if ws_bytes else None
     _lib.call("ody_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
               B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
               scale, int(causal), _dt(q), ws.data_ptr() if ws_bytes else 0, ws_bytes, _stream())
@@ -92,7 +109,7 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     lib = _lib.load()
     ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    ws = scratch(ws_bytes, "attn_bwd_workspace", q.device)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
     _lib.call("ody_attn_bwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
@@ -147,7 +164,7 @@ def gemm(op: int, a, b, bias=None, out=None, accumulate: bool = False):
     if bias is not None and (tuple(bias.shape) != (N,) or bias.dtype != a.dtype or not bias.is_contiguous()):
         raise ValueError(f"bias must be a contiguous ({N},) {a.dtype} tensor, got {tuple(bias.shape)} {bias.dtype}")
     ws_bytes = _lib.load().ody_gemm_workspace_bytes(op, M, N, K, _dt(a))
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    ws = scratch(ws_bytes, "gemm_workspace", a.device) if ws_bytes else None
     _lib.call("ody_gemm", op, a.data_ptr(), b.data_ptr(), out.data_ptr(), 0 if bias is None else bias.data_ptr(),
               M, N, K, _rowmajor2d(a, "a"), _rowmajor2d(b, "b"), _rowmajor2d(out, "out"),
               int(accumulate), _dt(a), ws.data_ptr() if ws is not None else 0, ws_bytes, _stream())
@@ -178,8 +195,47 @@ def swiglu_bwd(gate_up, dh):
     return dgu.view(gate_up.shape)
 
 
+def check_rmsnorm_args(x, weight, rstd=None, dy=None) -> None:
+    """The kernels read raw pointers: the weight must be a contiguous (d,) tensor of x's dtype on
+    x's device, dy must match x, rstd must hold one float32 per row."""
+    d = x.shape[-1]
+    if weight.dtype != x.dtype:
+        raise TypeError(f"rmsnorm: weight is {weight.dtype} but the activations are {x.dtype}; cast the module "
+                        "(`.to(dtype)`) so that both agree")
+    if tuple(weight.shape) != (d,) or not weight.is_contiguous() or weight.device != x.device:
+        raise ValueError(f"rmsnorm: weight must be a contiguous ({d},) tensor on {x.device}, got "
+                         f"{tuple(weight.shape)} on {weight.device}")
+    if dy is not None and (dy.dtype != x.dtype or dy.shape != x.shape or dy.device != x.device):
+        raise ValueError(f"rmsnorm: dy must match x ({tuple(x.shape)}, {x.dtype}, {x.device}); got "
+                         f"{tuple(dy.shape)}, {dy.dtype}, {dy.device}")
+    if rstd is not None:
+        rows = x.numel() // d if d else 0
+        if rstd.dtype != torch.float32 or rstd.numel() != rows or not rstd.is_contiguous() or rstd.device != x.device:
+            raise ValueError(f"rmsnorm: rstd must be a contiguous float32 tensor of {rows} rows on {x.device}; got "
+                             f"{tuple(rstd.shape)}, {rstd.dtype}, {rstd.device}")
+
+
+def check_rope_args(x, n_rot, position_ids, inv_freq) -> None:
+    B, L, H, D = x.shape
+    if not 0 <= n_rot <= H:
+        raise ValueError(f"n_rot={n_rot} exceeds the {H} heads of x")
+    if D % 2:
+        raise ValueError(f"rope: head_dim {D} is odd")
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or tuple(inv_freq.shape) != (D // 2,)
+                                 or not inv_freq.is_contiguous() or inv_freq.device != x.device):
+        raise ValueError(f"rope: inv_freq must be a contiguous float32 ({D // 2},) tensor on {x.device}; got "
+                         f"{tuple(inv_freq.shape)}, {inv_freq.dtype}, {inv_freq.device}")
+    if position_ids is not None:
+        if position_ids.dtype not in (torch.int64, torch.int32) or position_ids.device != x.device:
+            raise ValueError(f"rope: position_ids must be an integer tensor on {x.device}; got "
+                             f"{position_ids.dtype} on {position_ids.device}")
+        if position_ids.shape[-1] != L or position_ids.numel() not in (L, B * L):
+            raise ValueError(f"rope: position_ids {tuple(position_ids.shape)} do not cover (B={B}, L={L})")
+
+
 def rmsnorm_fwd(x, weight, eps: float = 1e-6):
     _need_gpu(x, weight)
+    check_rmsnorm_args(x, weight)
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
     T, d = x2.shape
     y = torch.empty_like(x2)
@@ -191,13 +247,14 @@ def rmsnorm_fwd(x, weight, eps: float = 1e-6):
 
 def rmsnorm_bwd(x, weight, rstd, dy):
     _need_gpu(x, weight, rstd, dy)
+    check_rmsnorm_args(x, weight, rstd, dy)
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
     dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
     T, d = x2.shape
     dx = torch.empty_like(x2)
     dw = torch.empty_like(weight)
     nparts = _lib.load().ody_rmsnorm_bwd_partials(T)
-    partial = torch.empty((nparts, d), dtype=torch.float32, device=x.device)
+    partial = scratch(nparts * d * 4, "rmsnorm_dw_partials", x.device)
     _lib.call("ody_rmsnorm_bwd", x2.data_ptr(), weight.data_ptr(), rstd.data_ptr(), dy2.data_ptr(), dx.data_ptr(),
               partial.data_ptr(), dw.data_ptr(), T, d, _dt(x2), _stream())
     return dx.view(x.shape), dw
@@ -220,10 +277,9 @@ def rope_(x, n_rot: int, position_ids=None, base: float = 10000.0, inverse: bool
     """Rotates heads [0, n_rot) of x (B, L, H, D) in place."""
     _need_gpu(x, position_ids, inv_freq)
     B, L, H, D = x.shape
-    if n_rot > H:
-        raise ValueError(f"n_rot={n_rot} exceeds the {H} heads of x")
     if inv_freq is None:
         inv_freq = rope_inv_freq(D, base, x.device)
+    check_rope_args(x, n_rot, position_ids, inv_freq)
     pos_ptr = 0
     if position_ids is not None:
         position_ids = position_ids.to(torch.int64).expand(B, L).contiguous()

@@ -1,0 +1,189 @@
+"""World-size-1 training step of the reference's driver (train.py:49-240) on one MI355X.
+
+    python -m odysseus_transformer_amd.train --use_cfg_init_model --parallel_mode odysseus
+
+Same measurement as the reference: `--max-train-steps` steps (10) on random token ids of
+`--seq-length` (16384) tokens, the first three untimed, memory printed after model and optimizer
+set-up and at every step, `loss.backward(loss)`, AdamW, and one line
+"<mode> <L/1024>K <world> Time taken: <s> seconds" at the end (train.py:167-235).  The model is the
+16-layer GQA 32/8 configuration of train.py:66-76, randomly initialised (no checkpoint can be
+fetched here; `--model` takes a local directory only), patched with
+apply_odysseus_attn_patch_llama / apply_tpsp_attn_patch_llama, with the loss from the fused
+cross-entropy kernel.
+
+What differs from the reference and why: one process, one GPU, no FSDP wrapping (its world-size-1
+branch skips it too, train.py:118); `--native-host-modules` (default on) also routes the host
+model's RMSNorms and lm_head through the HIP library, so that the step runs on this library's
+kernels except for the embedding lookup, the residual adds of the host decoder layer and the
+optimizer; switch it off to keep every host module as transformers ships it.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import time
+
+import torch
+from torch import nn
+
+
+class NativeLinear(nn.Module):
+    """Bias-free nn.Linear on the library's dense products (forward, dgrad, wgrad)."""
+
+    def __init__(self, linear: nn.Linear):
+        super().__init__()
+        if linear.bias is not None:
+            raise NotImplementedError("lm_head with a bias")
+        self.weight = linear.weight
+        self.in_features, self.out_features = linear.in_features, linear.out_features
+
+    def forward(self, x):
+        from .utils.linear_tpsp import _PlainLinearFunc
+        return _PlainLinearFunc.apply(x, self.weight)
+
+
+def use_native_host_modules(model) -> None:
+    """Swaps the host model's RMSNorm modules and lm_head for the library's (weights are shared)."""
+    from .decoder.odysseus import LlamaRMSNorm
+
+    def native_norm(old):
+        new = LlamaRMSNorm(old.weight.shape[0], getattr(old, "variance_epsilon", 1e-6))
+        new.weight = old.weight
+        return new
+
+    for layer in model.model.layers:
+        layer.input_layernorm = native_norm(layer.input_layernorm)
+        layer.post_attention_layernorm = native_norm(layer.post_attention_layernorm)
+    model.model.norm = native_norm(model.model.norm)
+    model.lm_head = NativeLinear(model.lm_head)
+
+
+def build_model(args, dev):
+    import transformers
+    from transformers import LlamaConfig
+    if args.use_cfg_init_model:
+        cfg = LlamaConfig()
+        cfg.hidden_size = 4096
+        cfg.intermediate_size = 11008
+        cfg.num_attention_heads = 32
+        cfg.num_key_value_heads = 8
+        cfg.num_hidden_layers = args.num_hidden_layers
+        cfg._attn_implementation = "flash_attention_2" if args.declare_flash_attention else "sdpa"
+        cfg.rope_theta = args.rope_theta
+        if hasattr(cfg, "rope_parameters") and isinstance(cfg.rope_parameters, dict):
+            cfg.rope_parameters["rope_theta"] = args.rope_theta
+        cfg.max_position_embeddings = max(getattr(cfg, "max_position_embeddings", 0) or 0, args.seq_length)
+        cfg.use_cache = False
+        with torch.device(dev):                       # initialise on the GPU: 3.1 B parameters take a minute on the host
+            model = transformers.LlamaForCausalLM(cfg).to(dtype=torch.bfloat16)
+    else:
+        import os
+        if not os.path.isdir(args.model):
+            raise SystemExit(f"--model {args.model!r} is not a local directory and nothing can be downloaded here; "
+                             "use --use_cfg_init_model")
+        model = transformers.AutoModelForCausalLM.from_pretrained(args.model, torch_dtype=torch.bfloat16)
+    return model
+
+
+def main(args) -> dict:
+    from .decoder.odysseus import apply_odysseus_attn_patch_llama
+    from .decoder.tensor_parallel import apply_tpsp_attn_patch_llama
+    from .losses.cross_entropy import CrossEntropyLoss
+    from .utils.apply_seq_parallel import prepare_attn_inputs
+    from .utils.globals import _Arena, _set_global_memory_buffer
+    from . import _lib
+
+    assert args.batch_size == 1, "Only support batch size 1"
+    rank, world_size = 0, 1
+    _lib.load()
+    torch.manual_seed(args.seed)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if _Arena.instance is None:
+        _set_global_memory_buffer(dev)
+
+    model = build_model(args, dev)
+    total_params = sum(p.numel() for p in model.parameters())
+    print(f"total parameters {total_params/1e9:.2f}B")
+    if args.parallel_mode == "odysseus":
+        print(f"use odysseus zero3 {args.use_ody_zero3}")
+        with torch.device(dev):
+            apply_odysseus_attn_patch_llama(model, use_zero3_linear=args.use_ody_zero3)
+    elif args.parallel_mode == "tpsp":
+        with torch.device(dev):
+            apply_tpsp_attn_patch_llama(model)
+    else:
+        raise SystemExit(f"parallel_mode {args.parallel_mode!r}: this build has the odysseus and tpsp modules "
+                         "(ulysses, ring and dp are collective choreography, which is out of its scope)")
+    model = model.to(dev)
+    from .utils.linear_zero3 import LinearZeRO3
+    with torch.no_grad():     # LinearZeRO3 leaves its weight uninitialised, as the reference does: give it finite values
+        for m in model.modules():
+            if isinstance(m, LinearZeRO3):
+                m.weight.normal_(0.0, 0.02)
+    if args.native_host_modules:
+        use_native_host_modules(model)
+    mem = lambda: (torch.cuda.memory_allocated(dev) / 1024 ** 3, torch.cuda.memory_reserved(dev) / 1024 ** 3)
+    print(f"{args.parallel_mode} After init model, CUDA memory allocated: {mem()[0]:.2f} GB, reserved: {mem()[1]:.2f} GB")
+
+    optim = torch.optim.AdamW(model.parameters(), lr=args.learning_rate)
+    model.train()
+    loss_func = CrossEntropyLoss(inplace_backward=True)
+    warmup_num_iterations = 2
+    elapse, step_times, losses = 0.0, [], []
+    print(f"{args.parallel_mode} After init optim, CUDA memory allocated: {mem()[0]:.2f} GB, reserved: {mem()[1]:.2f} GB")
+
+    gen = torch.Generator().manual_seed(args.seed)
+    vocab_size = model.config.vocab_size
+    for step in range(args.max_train_steps):
+        if step > warmup_num_iterations:
+            start_time = time.time()
+        batch = torch.randint(vocab_size, size=(1, args.seq_length + 1), generator=gen)
+        input_ids, target_ids = batch[..., :-1], batch[..., 1:]
+        position_ids = torch.arange(args.seq_length).unsqueeze(0).expand(input_ids.shape[0], -1)
+        prepared = prepare_attn_inputs(args.parallel_mode, input_ids, position_ids, target_ids, rank, world_size, dev)
+        logits = model(prepared["local_input_ids"], position_ids=prepared["local_position_ids"], use_cache=False).logits
+        loss = loss_func(logits.reshape(-1, logits.shape[-1]), prepared["local_target_ids"].reshape(-1))
+        print(f"step {step} CUDA memory allocated/reserved: {mem()[0]:.2f}/{mem()[1]:.2f} GB")
+        losses.append(loss.item())
+        print(f"loss {losses[-1]}", flush=True)
+        loss.backward(loss)
+        optim.step()
+        optim.zero_grad()
+        if step > warmup_num_iterations:
+            torch.cuda.synchronize()                  # the reference stops its clock without one; the next loss.item() pays for it there
+            step_times.append(time.time() - start_time)
+            elapse += step_times[-1]
+    print(f"{args.parallel_mode} {args.seq_length//1024}K {world_size} Time taken: {elapse:.2f} seconds")
+    out = {"parallel_mode": args.parallel_mode, "seq_length": args.seq_length, "layers": model.config.num_hidden_layers,
+           "parameters_b": round(total_params / 1e9, 3), "timed_steps": len(step_times), "time_taken_s": round(elapse, 3),
+           "step_ms": [round(1e3 * t, 1) for t in step_times], "tokens_per_s": round(args.seq_length * len(step_times) /
+                                                                                      max(elapse, 1e-9), 1),
+           "peak_memory_gb": round(torch.cuda.max_memory_allocated(dev) / 1024 ** 3, 2), "losses": [round(l, 4) for l in losses],
+           "native_host_modules": bool(args.native_host_modules)}
+    print(json.dumps(out))
+    return out
+
+
+def parse_args(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--batch-size", type=int, default=1)
+    ap.add_argument("--seed", type=int, default=42)
+    ap.add_argument("--max-train-steps", type=int, default=10)
+    ap.add_argument("--learning-rate", type=float, default=2e-5)
+    ap.add_argument("--rope-theta", type=float, default=100000)
+    ap.add_argument("--model", type=str, default="meta-llama/Llama-2-7b-hf")
+    ap.add_argument("--seq-length", type=int, default=16384)
+    ap.add_argument("--use_ody_zero3", action="store_true", default=True)
+    ap.add_argument("--use_cfg_init_model", action="store_true", default=False)
+    ap.add_argument("--parallel_mode", type=str, choices=["odysseus", "ulysses", "dp", "tpsp", "ring"], default="odysseus")
+    ap.add_argument("--num-hidden-layers", type=int, default=16, help="16 in the reference's configuration (train.py:71)")
+    ap.add_argument("--native-host-modules", action=argparse.BooleanOptionalAction, default=True)
+    ap.add_argument("--declare-flash-attention", action=argparse.BooleanOptionalAction, default=False,
+                    help="set config._attn_implementation before the model is built (needs flash_attn importable); "
+                         "the patchers set it afterwards either way")
+    return ap.parse_args(argv)
+
+
+if __name__ == "__main__":
+    main(parse_args())

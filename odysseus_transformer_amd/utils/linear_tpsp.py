@@ -71,6 +71,16 @@ def allgather_along_first_dim_from_model_parallel_region(input_: torch.Tensor) -
 
 
 # ---------------------------------------------------------------- the three products
+def _autocast(*ts):
+    """What torch.matmul does under autocast, which the reference relies on through custom_fwd /
+    custom_bwd (utils/linear_tpsp.py:129,180, utils/linear_zero3.py:24,51): operands are cast to
+    the autocast dtype.  Outside autocast the tensors pass through and a dtype mismatch raises."""
+    if torch.is_autocast_enabled("cuda"):
+        dt = torch.get_autocast_dtype("cuda")
+        return tuple(t if t is None or t.dtype == dt else t.to(dt) for t in ts)
+    return ts
+
+
 def _as_2d(t: torch.Tensor) -> torch.Tensor:
     t2 = t.reshape(-1, t.shape[-1])
     return t2 if t2.stride(-1) == 1 else t2.contiguous()
@@ -79,6 +89,7 @@ def _as_2d(t: torch.Tensor) -> torch.Tensor:
 def linear_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     """Y = X W^T (+ b) over the last dimension of x.  The result is allocated in its final
     shape (not returned as a view), so that a following in-place op may own it."""
+    x, weight, bias = _autocast(x, weight, bias)
     y = torch.empty((*x.shape[:-1], weight.shape[0]), dtype=x.dtype, device=x.device)
     ops.gemm(ops.GEMM_NT, _as_2d(x), weight, bias=bias, out=y.view(-1, weight.shape[0]))
     return y
@@ -86,6 +97,7 @@ def linear_forward(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
 
 def linear_dgrad(grad_output: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """dX = dY W."""
+    grad_output, weight = _autocast(grad_output, weight)
     dx = torch.empty((*grad_output.shape[:-1], weight.shape[1]), dtype=grad_output.dtype, device=grad_output.device)
     ops.gemm(ops.GEMM_NN, _as_2d(grad_output), weight, out=dx.view(-1, weight.shape[1]))
     return dx
@@ -93,6 +105,7 @@ def linear_dgrad(grad_output: torch.Tensor, weight: torch.Tensor) -> torch.Tenso
 
 def linear_wgrad(grad_output_2d: torch.Tensor, input_2d: torch.Tensor) -> torch.Tensor:
     """dW = dY^T X on the flattened, contiguous pair."""
+    grad_output_2d, input_2d = _autocast(grad_output_2d, input_2d)
     return ops.gemm(ops.GEMM_TN, grad_output_2d, input_2d)
 
 
@@ -102,6 +115,7 @@ class LinearWithGradAccumulationAndAsyncCommunication(torch.autograd.Function):
     saved; backward re-gathers the input."""
 
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, input, weight, bias, gradient_accumulation_fusion, async_grad_allreduce, sequence_parallel,
                 grad_output_buffer):
         ctx.save_for_backward(input, weight)
@@ -119,6 +133,7 @@ class LinearWithGradAccumulationAndAsyncCommunication(torch.autograd.Function):
         return linear_forward(total_input, weight, bias)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
         wgrad_compute = True
@@ -192,9 +207,11 @@ def _init_partitioned_weight(weight, out_features, in_features, per_partition, p
     return master if return_master_weight else None
 
 
-class ColumnParallelLinearAG(torch.nn.Module):
-    """Y = gather(X) A_i^T: the weight is split along its OUTPUT rows, the input is the
-    sequence shard and is gathered inside (utils/linear_tpsp.py:405-500)."""
+class _ColumnParallelLinearBase(torch.nn.Module):
+    """Y = X A_i^T: the weight is split along its OUTPUT rows.  The two public classes differ in one
+    flag only: whether the input is the sequence shard that the layer gathers itself."""
+
+    sequence_parallel: bool = False
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, gather_output: bool = True,
                  init_method: Callable[[torch.Tensor], torch.Tensor] = init.xavier_normal_, stride: int = 1,
@@ -221,46 +238,25 @@ class ColumnParallelLinearAG(torch.nn.Module):
     def forward(self, input_: torch.Tensor) -> torch.Tensor:
         output_parallel = linear_with_grad_accumulation_and_async_allreduce(
             input=input_, weight=self.weight, bias=self.bias, gradient_accumulation_fusion=False,
-            async_grad_allreduce=False, sequence_parallel=True)
+            async_grad_allreduce=False, sequence_parallel=self.sequence_parallel)
         if self.gather_output:
             require_single_rank("gather of the column-split output")
         return output_parallel
 
 
-class ColumnParallelLinear(torch.nn.Module):
+class ColumnParallelLinearAG(_ColumnParallelLinearBase):
+    """Y = gather(X) A_i^T: the input is the sequence shard and is gathered inside
+    (utils/linear_tpsp.py:405-500)."""
+
+    sequence_parallel = True
+
+
+class ColumnParallelLinear(_ColumnParallelLinearBase):
     """Column-split linear WITHOUT the sequence gather: the unpacked q/k/v branch and the
     non-sequence-parallel branch of the attention block (decoder/odysseus.py:96-137) take
     it from fairscale; the caller gathers the sequence first."""
 
-    def __init__(self, in_features: int, out_features: int, bias: bool = True, gather_output: bool = True,
-                 init_method: Callable[[torch.Tensor], torch.Tensor] = init.xavier_normal_, stride: int = 1,
-                 keep_master_weight_for_test: bool = False) -> None:
-        super().__init__()
-        self.in_features = in_features
-        self.out_features = out_features
-        self.gather_output = gather_output
-        world_size = get_model_parallel_world_size()
-        self.output_size_per_partition = divide_and_check_no_remainder(out_features, world_size)
-        self.weight = Parameter(torch.empty(self.output_size_per_partition, self.in_features))
-        if bias:
-            self.bias = Parameter(torch.zeros(self.output_size_per_partition))
-        else:
-            self.register_parameter("bias", None)
-        self.master_weight = _init_partitioned_weight(
-            self.weight, self.out_features, self.in_features, self.output_size_per_partition, 0, init_method,
-            stride=stride, return_master_weight=keep_master_weight_for_test)
-
-    def get_master_weight(self) -> torch.Tensor:
-        require_single_rank("gather of the column-split weight")
-        return self.weight.data.clone()
-
-    def forward(self, input_: torch.Tensor) -> torch.Tensor:
-        output_parallel = linear_with_grad_accumulation_and_async_allreduce(
-            input=input_, weight=self.weight, bias=self.bias, gradient_accumulation_fusion=False,
-            async_grad_allreduce=False, sequence_parallel=False)
-        if self.gather_output:
-            require_single_rank("gather of the column-split output")
-        return output_parallel
+    sequence_parallel = False
 
 
 class _PlainLinearFunc(torch.autograd.Function):
@@ -268,11 +264,13 @@ class _PlainLinearFunc(torch.autograd.Function):
     the backward autograd derives for it)."""
 
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, input, weight):
         ctx.save_for_backward(input, weight)
         return linear_forward(input, weight, None)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
         grad_input = linear_dgrad(grad_output, weight)

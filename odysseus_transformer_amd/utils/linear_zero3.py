@@ -31,12 +31,14 @@ def _reduce_scatter_weight_grad(grad_weight_global: torch.Tensor) -> torch.Tenso
 
 class LinearZeROFunc(torch.autograd.Function):
     @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda")
     def forward(ctx, input, weight, bias):
         ctx.save_for_backward(input, weight)
         ctx.use_bias = bias is not None
         return linear_forward(input, _gather_weight(weight), bias)
 
     @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
         input, weight = ctx.saved_tensors
         full_weight = _gather_weight(weight)

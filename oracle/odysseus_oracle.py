@@ -31,6 +31,8 @@ How each function is pinned (tests/test_oracle.py):
   linear_*           == torch.nn.functional.linear + autograd in fp64
   swiglu_mlp_*       == silu(x Wg^T) * (x Wu^T) then Wd, the HF LlamaMLP
                      formula with gate = W[:i], up = W[i:]
+  cross_entropy_*    == torch.nn.functional.cross_entropy (mean, ignore_index) and its
+                     autograd gradient in fp64; rows of the gradient sum to zero
   attention_block,   autograd of the composed functions vs. the explicit
   decoder_layer_*    backward formulas in this file
 
@@ -313,6 +315,26 @@ def swiglu_mlp_bwd(x, w_gate_up, w_down, dy):
     dgu = swiglu_bwd(gu, dh)
     dx, dwgu, _ = linear_bwd(x, w_gate_up, dgu)
     return dx, dwgu, dwd
+
+
+# --------------------------------------------------------------------------
+# Cross-entropy  (train.py:173,212-214: flash_attn's CrossEntropyLoss on logits (T, V) and
+# labels (T); mean over the tokens whose label is not ignore_index)
+# --------------------------------------------------------------------------
+def cross_entropy_fwd_bwd(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100,
+                          grad_loss: float = 1.0):
+    """Returns (mean loss, per-token losses, lse, d mean-loss / d logits * grad_loss)."""
+    ct = _ct(logits)
+    x = logits.to(ct)
+    lse = torch.logsumexp(x, dim=-1)
+    valid = labels != ignore_index
+    safe = torch.where(valid, labels, torch.zeros_like(labels))
+    losses = torch.where(valid, lse - x.gather(1, safe[:, None])[:, 0], torch.zeros_like(lse))
+    n = valid.sum().clamp_min(1).to(ct)
+    p = torch.exp(x - lse[:, None])
+    onehot = torch.zeros_like(p).scatter_(1, safe[:, None], 1.0)
+    dlogits = (p - onehot) * valid[:, None].to(ct) * (grad_loss / n)
+    return losses.sum() / n, losses, lse, dlogits
 
 
 # --------------------------------------------------------------------------

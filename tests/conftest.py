@@ -39,6 +39,52 @@ def rel_err(a: torch.Tensor, ref: torch.Tensor, floor: float = 1e-3) -> float:
     return (a - ref).abs().max().item() / den
 
 
+def block_rel_err(a: torch.Tensor, ref: torch.Tensor, floor: float = 1e-3, floor_frac: float = 1e-3,
+                  seq_dim=None, block: int = 64) -> float:
+    """Largest BLOCK-WISE relative error: the tensor is cut along its sequence dimension into blocks
+    of `block` consecutive positions (separately for every batch entry and head); for each block,
+    max |a - ref| over the block divided by max |ref| over the same block.
+
+    Under a causal mask the rows of out / dq / dk / dv shrink like 1 / sqrt(position), so a
+    whole-tensor normalisation is set by the first rows and says little about the rest of a long
+    sequence: a result whose second half is missing passes it.  This metric holds every block of
+    64 rows to the tolerance on the block's own scale.  It is not taken row by row because single
+    rows can be ill-conditioned: a query whose softmax sits on one key has dS = P (dP - delta) ~ 0
+    by cancellation, and the bf16 rounding of `out` that every flash-attention backward inherits
+    through delta = sum(dO * out) then is 10 % of that row (measured on an exact-arithmetic
+    emulation with only `out` rounded).  A block of neighbouring rows is not.
+
+    seq_dim: the dimension along which rows are neighbours (default: 1 for (B, L, H, D), 0 for
+    (L, H, D) and for matrices).  The denominator is floored at `floor_frac` of the tensor's
+    largest magnitude and at `floor` (the same absolute floor as rel_err)."""
+    a, ref = a.detach().double().cpu(), ref.detach().double().cpu()
+    if ref.numel() == 0:
+        return 0.0
+    if ref.dim() < 2:
+        return rel_err(a, ref, floor)
+    if seq_dim is None:
+        seq_dim = 1 if ref.dim() == 4 else 0
+    err = (a - ref).abs().amax(-1).movedim(seq_dim, -1)        # (..., L)
+    mag = ref.abs().amax(-1).movedim(seq_dim, -1)
+    L = err.shape[-1]
+    pad = (-L) % block
+    if pad:
+        err = torch.nn.functional.pad(err, (0, pad))
+        mag = torch.nn.functional.pad(mag, (0, pad))
+    err = err.reshape(*err.shape[:-1], -1, block).amax(-1)
+    mag = mag.reshape(*mag.shape[:-1], -1, block).amax(-1)
+    den = mag.clamp_min(max(floor_frac * ref.abs().max().item(), floor))
+    return (err / den).max().item()
+
+
+def assert_parity(a: torch.Tensor, ref: torch.Tensor, tol: float, what: str = "", floor: float = 1e-3,
+                  seq_dim=None, block: int = 64) -> None:
+    """The parity bar: whole-tensor AND block-wise relative error within `tol`."""
+    g, r = rel_err(a, ref, floor), block_rel_err(a, ref, floor, seq_dim=seq_dim, block=block)
+    assert g <= tol, f"{what}: whole-tensor relative error {g:.3e} > {tol}"
+    assert r <= tol, f"{what}: block-wise relative error {r:.3e} > {tol}"
+
+
 def randn(shape, seed, std=1.0, dtype=torch.float32):
     g = torch.Generator(device="cpu").manual_seed(seed)
     return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(dtype)

@@ -4,7 +4,7 @@ import math
 import pytest
 import torch
 
-from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
+from conftest import TOL_BF16, TOL_F32, TOL_LSE, assert_parity, randn, rel_err
 import odysseus_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -47,15 +47,15 @@ def test_attention_fwd_bwd(case, dtype, dev):
     qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
     o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
     torch.cuda.synchronize()
-    assert rel_err(o, o_ref) <= tol
+    assert_parity(o, o_ref, tol, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
     dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal)
     torch.cuda.synchronize()
     # with a single key dS = P (dP - delta) is identically zero: compare on the scale of the inputs
     floor = 1.0 if Lk == 1 else 1e-3
-    assert rel_err(dq, dq_ref, floor) <= tol, "dq"
-    assert rel_err(dk, dk_ref, floor) <= tol, "dk"
-    assert rel_err(dv, dv_ref) <= tol, "dv"
+    assert_parity(dq, dq_ref, tol, "dq", floor)
+    assert_parity(dk, dk_ref, tol, "dk", floor)
+    assert_parity(dv, dv_ref, tol, "dv")
 
 
 def test_attention_strided_views_of_packed_qkv(dev):
@@ -69,7 +69,7 @@ def test_attention_strided_views_of_packed_qkv(dev):
     qg, kg, vg = g[:, :, :Hq], g[:, :, Hq:Hq + Hkv], g[:, :, Hq + Hkv:]
     assert not qg.is_contiguous()
     o, lse = ops.attn_fwd(qg, kg, vg, causal=True)
-    assert rel_err(o, o_ref) <= TOL_BF16
+    assert_parity(o, o_ref, TOL_BF16, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
     # gradients written straight into a packed dqkv buffer
     do = randn((B, L, Hq, D), 6, dtype=torch.bfloat16)
@@ -77,9 +77,9 @@ def test_attention_strided_views_of_packed_qkv(dev):
     dqkv = torch.zeros_like(g)
     ops.attn_bwd(qg, kg, vg, o, lse, do.to(dev), dq=dqkv[:, :, :Hq], dk=dqkv[:, :, Hq:Hq + Hkv],
                  dv=dqkv[:, :, Hq + Hkv:])
-    assert rel_err(dqkv[:, :, :Hq], dq_ref) <= TOL_BF16
-    assert rel_err(dqkv[:, :, Hq:Hq + Hkv], dk_ref) <= TOL_BF16
-    assert rel_err(dqkv[:, :, Hq + Hkv:], dv_ref) <= TOL_BF16
+    assert_parity(dqkv[:, :, :Hq], dq_ref, TOL_BF16, "dq")
+    assert_parity(dqkv[:, :, Hq:Hq + Hkv], dk_ref, TOL_BF16, "dk")
+    assert_parity(dqkv[:, :, Hq + Hkv:], dv_ref, TOL_BF16, "dv")
 
 
 def test_attention_row_properties(dev):
@@ -100,7 +100,7 @@ def test_attention_row_properties(dev):
         ref_lse = torch.logsumexp(s, -1)
         ref_o = torch.softmax(s, -1) @ v[0, :, h].double()
         assert torch.allclose(lse[0, h, rows].cpu().double(), ref_lse, atol=TOL_LSE, rtol=TOL_LSE)
-        assert rel_err(o[0, rows, h], ref_o) <= TOL_BF16
+        assert_parity(o[0, rows, h], ref_o, TOL_BF16, f"out head {h}")
 
 
 def test_attention_scores_beyond_the_reference_window(dev):
@@ -119,10 +119,16 @@ def test_attention_scores_beyond_the_reference_window(dev):
     qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
     o, lse = ops.attn_fwd(qg, kg, vg, causal=True)
     assert torch.isfinite(o).all() and torch.isfinite(lse).all()
-    assert rel_err(o, o_ref) <= TOL_BF16
+    assert_parity(o, o_ref, TOL_BF16, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
     dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True)
+    # head 0 is built to be degenerate: every query's softmax sits on a handful of keys, so its dS
+    # is small by cancellation in whole blocks of rows; the gradients are held to the scale of the
+    # tensor here, and to the scale of their own block in every other test
     assert rel_err(dq, dq_ref) <= TOL_BF16 and rel_err(dk, dk_ref) <= TOL_BF16 and rel_err(dv, dv_ref) <= TOL_BF16
+    assert_parity(dq[:, :, 1:], dq_ref[:, :, 1:], TOL_BF16, "dq of the ordinary head")
+    assert_parity(dk[:, :, 1:], dk_ref[:, :, 1:], TOL_BF16, "dk of the ordinary head")
+    assert_parity(dv[:, :, 1:], dv_ref[:, :, 1:], TOL_BF16, "dv of the ordinary head")
 
 
 def test_attention_errors(dev):
@@ -167,11 +173,11 @@ def test_attention_random_shapes(case, dev):
     o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
     dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal)
     floor = 1.0 if Lk == 1 else 1e-3
-    assert rel_err(o, o_ref) <= TOL_BF16
+    assert_parity(o, o_ref, TOL_BF16, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
-    assert rel_err(dq, dq_ref, floor) <= TOL_BF16, "dq"
-    assert rel_err(dk, dk_ref, floor) <= TOL_BF16, "dk"
-    assert rel_err(dv, dv_ref) <= TOL_BF16, "dv"
+    assert_parity(dq, dq_ref, TOL_BF16, "dq", floor)
+    assert_parity(dk, dk_ref, TOL_BF16, "dk", floor)
+    assert_parity(dv, dv_ref, TOL_BF16, "dv")
 
 
 @pytest.mark.parametrize("D", [64, 128])
@@ -190,8 +196,8 @@ def test_attention_random_shapes_fp32(case, D, dev):
     dq = dq0.clone()
     _, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=dq, accumulate_dq=True)
     floor = 1.0 if Lk == 1 else 1e-3
-    assert rel_err(o, o_ref) <= TOL_F32
+    assert_parity(o, o_ref, TOL_F32, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
-    assert rel_err(dq - dq0, dq_ref, floor) <= 4 * TOL_F32, "dq"      # the difference of two rounded sums
-    assert rel_err(dk, dk_ref, floor) <= TOL_F32, "dk"
-    assert rel_err(dv, dv_ref) <= TOL_F32, "dv"
+    assert_parity(dq - dq0, dq_ref, 4 * TOL_F32, "dq", floor)  # the difference of two rounded sums
+    assert_parity(dk, dk_ref, TOL_F32, "dk", floor)
+    assert_parity(dv, dv_ref, TOL_F32, "dv")

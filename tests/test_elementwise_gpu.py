@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
+from conftest import TOL_BF16, TOL_F32, TOL_LSE, assert_parity, randn, rel_err
 import odysseus_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -129,7 +129,7 @@ def test_ring_step_equals_unsplit_attention(dev):
     for b in range(NB):
         ob, lb = ops.attn_fwd(qg, ks[b].to(dev), vs[b].to(dev), causal=(b == 0))
         ops.lse_merge_(out, lse, ob, lb)
-    assert rel_err(out, o_ref) <= TOL_BF16
+    assert_parity(out, o_ref, TOL_BF16, "out")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
     out_bf = out.to(dt)
     dq = torch.zeros_like(qg)
@@ -139,9 +139,9 @@ def test_ring_step_equals_unsplit_attention(dev):
                                  accumulate_dq=(b > 0))
         dks.append(dk)
         dvs.append(dv)
-    assert rel_err(dq, dq_ref) <= TOL_BF16
-    assert rel_err(torch.cat(dks[1:] + dks[:1], 1), dk_ref) <= TOL_BF16
-    assert rel_err(torch.cat(dvs[1:] + dvs[:1], 1), dv_ref) <= TOL_BF16
+    assert_parity(dq, dq_ref, TOL_BF16, "dq")
+    assert_parity(torch.cat(dks[1:] + dks[:1], 1), dk_ref, TOL_BF16, "dk")
+    assert_parity(torch.cat(dvs[1:] + dvs[:1], 1), dv_ref, TOL_BF16, "dv")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
@@ -162,7 +162,9 @@ def test_ring_blocks_autograd_function(dtype, dev):
     vg = [t.to(dev).requires_grad_() for t in vs]
     out, lse = ops.ring_blocks_attn(qg, kg, vg, causal_block=1)
     out.backward(do.to(dev))
-    assert rel_err(out, o_ref) <= tol and torch.allclose(lse.cpu(), l_ref, atol=TOL_LSE, rtol=TOL_LSE)
-    assert rel_err(qg.grad, dq_ref) <= tol
+    assert_parity(out, o_ref, tol, "out")
+    assert torch.allclose(lse.cpu(), l_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    assert_parity(qg.grad, dq_ref, tol, "dq")
     for b in range(NB):
-        assert rel_err(kg[b].grad, dk_ref[b]) <= tol and rel_err(vg[b].grad, dv_ref[b]) <= tol
+        assert_parity(kg[b].grad, dk_ref[b], tol, f"dk block {b}")
+        assert_parity(vg[b].grad, dv_ref[b], tol, f"dv block {b}")

@@ -183,3 +183,95 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
+
+
+# ------------------------------------------------------------------ argument checks of the op wrappers
+def test_rmsnorm_and_rope_wrappers_check_what_the_kernels_cannot():
+    from odysseus_transformer_amd import ops
+    x = torch.zeros(4, 16, dtype=torch.bfloat16)
+    ops.check_rmsnorm_args(x, torch.ones(16, dtype=torch.bfloat16))
+    with pytest.raises(TypeError, match="weight is torch.float32"):
+        ops.check_rmsnorm_args(x, torch.ones(16))                      # fp32 weight, bf16 activations
+    with pytest.raises(ValueError, match="weight must be"):
+        ops.check_rmsnorm_args(x, torch.ones(8, dtype=torch.bfloat16))  # too short: the kernel would read past it
+    with pytest.raises(ValueError, match="weight must be"):
+        ops.check_rmsnorm_args(x, torch.ones(32, dtype=torch.bfloat16)[::2])
+    with pytest.raises(ValueError, match="dy must match"):
+        ops.check_rmsnorm_args(x, torch.ones(16, dtype=torch.bfloat16), torch.ones(4), torch.zeros(4, 16))
+    with pytest.raises(ValueError, match="rstd must be"):
+        ops.check_rmsnorm_args(x, torch.ones(16, dtype=torch.bfloat16), torch.ones(3), x)
+    with pytest.raises(ValueError, match="rstd must be"):
+        ops.check_rmsnorm_args(x, torch.ones(16, dtype=torch.bfloat16), torch.ones(4, dtype=torch.float64), x)
+    q = torch.zeros(1, 8, 3, 16)
+    ops.check_rope_args(q, 2, torch.arange(8)[None], torch.ones(8))
+    with pytest.raises(ValueError, match="exceeds"):
+        ops.check_rope_args(q, 4, None, None)
+    with pytest.raises(ValueError, match="inv_freq must be"):
+        ops.check_rope_args(q, 2, None, torch.ones(4))
+    with pytest.raises(ValueError, match="inv_freq must be"):
+        ops.check_rope_args(q, 2, None, torch.ones(8, dtype=torch.float64))
+    with pytest.raises(ValueError, match="position_ids must be"):
+        ops.check_rope_args(q, 2, torch.zeros(1, 8), None)
+    with pytest.raises(ValueError, match="do not cover"):
+        ops.check_rope_args(q, 2, torch.arange(7)[None], None)
+    with pytest.raises(RuntimeError, match="only on a HIP device"):    # and no CPU fallback behind the checks
+        ops.rmsnorm_fwd(x, torch.ones(16, dtype=torch.bfloat16))
+
+
+def test_scratch_comes_from_the_arena_when_it_is_set_up():
+    from odysseus_transformer_amd import ops
+    g._destroy_global_memory_buffer()
+    cpu = torch.device("cpu")
+    a = ops.scratch(1000, "attn_fwd_workspace", cpu)
+    b = ops.scratch(1000, "attn_fwd_workspace", cpu)
+    assert a.data_ptr() != b.data_ptr() or a.data_ptr() == 0          # no arena: fresh allocations
+    g._set_global_memory_buffer("cpu")
+    try:
+        a = ops.scratch(1000, "attn_fwd_workspace", cpu)
+        b = ops.scratch(600, "attn_fwd_workspace", cpu)
+        c = ops.scratch(600, "attn_bwd_workspace", cpu)
+        assert a.data_ptr() == b.data_ptr() and c.data_ptr() != a.data_ptr()
+        assert a.numel() == 1000 and b.numel() == 600 and a.dtype == torch.uint8
+        big = ops.scratch(5000, "attn_fwd_workspace", cpu)                # grows, then stays
+        assert ops.scratch(1000, "attn_fwd_workspace", cpu).data_ptr() == big.data_ptr()
+        # an arena of another device type is not used
+        assert ops.scratch(10, "x", torch.device("meta")).device.type == "meta"
+    finally:
+        g._destroy_global_memory_buffer()
+
+
+def test_patchers_stop_the_host_from_building_dense_masks():
+    """With attn_implementation='eager' transformers passes a dense causal mask to every layer,
+    which the modules refuse; after the patch the forward reaches the ops (which refuse CPU tensors)."""
+    transformers = pytest.importorskip("transformers")
+    from odysseus_transformer_amd.decoder.odysseus import apply_odysseus_attn_patch_llama
+    from odysseus_transformer_amd.decoder.tensor_parallel import LlamaMLPTPSP, apply_tpsp_attn_patch_llama
+    for patch in (apply_odysseus_attn_patch_llama, apply_tpsp_attn_patch_llama):
+        cfg = transformers.LlamaConfig(hidden_size=64, intermediate_size=96, num_hidden_layers=2, num_attention_heads=2,
+                                       num_key_value_heads=1, head_dim=32, vocab_size=64)
+        cfg._attn_implementation = "eager"
+        model = transformers.LlamaForCausalLM(cfg)
+        patch(model)
+        assert model.config._attn_implementation == "flash_attention_2"
+        with pytest.raises(RuntimeError, match="only on a HIP device"):
+            model(torch.randint(0, 64, (1, 16)), position_ids=torch.arange(16)[None])
+    assert isinstance(model.model.layers[0].mlp, LlamaMLPTPSP)
+    assert tuple(model.model.layers[1].mlp.w1w3.weight.shape) == (192, 64)
+    assert tuple(model.model.layers[1].mlp.w2.weight.shape) == (64, 96)
+
+
+def test_tpsp_mlp_surface():
+    from odysseus_transformer_amd.decoder.tensor_parallel import LlamaMLPTPSP
+    from odysseus_transformer_amd.utils.linear_tpsp import ColumnParallelLinear, ColumnParallelLinearAG, RowParallelLinearRS
+    m = LlamaMLPTPSP(_cfg())
+    assert isinstance(m.w1w3, ColumnParallelLinearAG) and isinstance(m.w2, RowParallelLinearRS)
+    assert m.w1w3.bias is None and m.w2.bias is None and m.w2.input_is_parallel
+    m = LlamaMLPTPSP(_cfg(), pack_weight=True, sequence_parallel=False, keep_master_weight_for_test=True)
+    assert type(m.w1w3) is ColumnParallelLinear and m.w1w3.master_weight is not None
+    m = LlamaMLPTPSP(_cfg(), pack_weight=False)
+    assert type(m.w1) is ColumnParallelLinear and tuple(m.w1.weight.shape) == (96, 64) and not hasattr(m, "w1w3")
+    ps.initialize_model_parallel(4, 1)
+    m = LlamaMLPTPSP(_cfg())
+    assert tuple(m.w1w3.weight.shape) == (48, 64) and tuple(m.w2.weight.shape) == (64, 24)
+    with pytest.raises(AssertionError, match="Pretraining TP"):
+        LlamaMLPTPSP(_cfg(pretraining_tp=2))(torch.zeros(1, 4, 64))

@@ -187,3 +187,74 @@ def test_layer_step_replayed_from_a_hip_graph(case, dev):
         for got, want in zip(captured, eager):
             assert torch.equal(got, want), f"replay {replay} differs from the eager step"
         float(torch.randn(4096, device=dev).square().sum())   # eager work and a synchronisation between replays
+
+
+def test_scratch_arena_removes_the_workspace_allocations(dev):
+    """With the process-wide arena set up (utils/globals.py, as train.py:62 of the reference does),
+    attention, split-K GEMM and RMSNorm scratch comes from its grow-only buffers: a layer step
+    makes fewer allocator requests than without it, the buffers keep their addresses from step to
+    step, and the results do not change."""
+    from odysseus_transformer_amd.decoder.odysseus import OdysseusDecoderLayer
+    from odysseus_transformer_amd.utils import globals as g
+    name, L, d, H, Hkv, D, i, dtype = LAYER_CASES[1]
+    layer = _load(OdysseusDecoderLayer(_config(d, H, Hkv, D, i)).to(dtype), _params(d, H, Hkv, D, i, dtype), dev)
+    x = randn((1, L, d), 41, dtype=dtype).to(dev).requires_grad_(True)
+    dy = randn((1, L, d), 42, dtype=dtype).to(dev)
+    pos = torch.arange(L, device=dev)[None]
+
+    def step():
+        for t in list(layer.parameters()) + [x]:
+            t.grad = None
+        y = layer(x, position_ids=pos)
+        y.backward(dy)
+        torch.cuda.synchronize()
+        return [y.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in layer.parameters()]
+
+    def counted(fn):
+        a0 = torch.cuda.memory_stats()["allocation.all.allocated"]
+        out = fn()
+        return out, torch.cuda.memory_stats()["allocation.all.allocated"] - a0
+
+    g._destroy_global_memory_buffer()
+    step()
+    plain, n_plain = counted(step)
+    g._set_global_memory_buffer(dev)
+    try:
+        step()                                       # the arena grows to its steady size here
+        ptrs = {k: v.data_ptr() for k, v in g.get_global_memory_buffer().buffer.items()}
+        assert {k[0] for k in ptrs} >= {"attn_fwd_workspace", "attn_bwd_workspace", "rmsnorm_dw_partials"}
+        with_arena, n_arena = counted(step)
+        _, n_arena2 = counted(step)
+        assert {k: v.data_ptr() for k, v in g.get_global_memory_buffer().buffer.items()} == ptrs
+        assert n_arena == n_arena2 and n_arena <= n_plain - 4, (n_plain, n_arena)   # fwd ws, bwd ws, 2 x norm partials
+        for a, b in zip(plain, with_arena):
+            assert torch.equal(a, b)
+    finally:
+        g._destroy_global_memory_buffer()
+
+
+def test_linears_follow_autocast(dev):
+    """fp32 modules under torch.autocast(bfloat16): the products run in bf16 as torch.matmul would
+    (the reference's custom_fwd / custom_bwd, utils/linear_tpsp.py:129,180), outputs are bf16 and
+    the weight gradients arrive in the parameters' fp32."""
+    from odysseus_transformer_amd.utils.linear_tpsp import ColumnParallelLinearAG, RowParallelLinearRS
+    from odysseus_transformer_amd.utils.linear_zero3 import LinearZeRO3
+    x = randn((1, 256, 512), 51).to(dev).requires_grad_(True)
+    w = randn((768, 512), 52, std=0.02)
+    for make in (lambda: ColumnParallelLinearAG(512, 768, bias=False, gather_output=False),
+                 lambda: RowParallelLinearRS(512, 768, bias=False, input_is_parallel=True),
+                 lambda: LinearZeRO3(512, 768)):
+        m = make().to(dev)
+        with torch.no_grad():
+            m.weight.copy_(w)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = m(x)
+        assert y.dtype == torch.bfloat16
+        y.float().sum().backward()
+        assert m.weight.grad.dtype == torch.float32 and x.grad.dtype == torch.float32
+        y_ref = oracle.linear_fwd(x.detach().cpu().bfloat16().float(), w.bfloat16().float())
+        assert rel_err(y, y_ref) <= TOL_BF16
+        assert rel_err(m.weight.grad, x.detach().cpu()[0].sum(0)[None].expand(768, 512)) <= TOL_BF16
+        with pytest.raises(TypeError):               # outside autocast a dtype mismatch still raises
+            m(x.bfloat16())

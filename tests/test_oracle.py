@@ -287,3 +287,20 @@ def test_sampled_checker_accepts_the_oracle_and_rejects_mistakes(Hq, Hkv, Lq, Lk
         wrong[idx] = bad
         with pytest.raises(AssertionError):
             sampled_checks(*wrong, True, rows, cols)
+
+
+def test_cross_entropy_equals_torch_and_its_autograd():
+    g = torch.Generator().manual_seed(5)
+    T, V = 37, 101
+    x = torch.randn(T, V, generator=g, dtype=torch.float64) * 3
+    y = torch.randint(0, V, (T,), generator=g)
+    y[::5] = -100
+    loss, losses, lse, dx = oracle.cross_entropy_fwd_bwd(x, y, grad_loss=0.7)
+    xr = x.clone().requires_grad_(True)
+    ref = torch.nn.functional.cross_entropy(xr, y, ignore_index=-100)
+    (ref * 0.7).backward()
+    assert torch.allclose(loss, ref.detach(), rtol=1e-12)
+    assert torch.allclose(dx, xr.grad, rtol=1e-10, atol=1e-14)
+    assert torch.allclose(losses, torch.nn.functional.cross_entropy(x, y, ignore_index=-100, reduction="none"), rtol=1e-12)
+    assert torch.allclose(lse, torch.logsumexp(x, -1))
+    assert dx.sum(-1).abs().max() < 1e-12 and (dx[::5] == 0).all()
