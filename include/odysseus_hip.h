@@ -96,6 +96,27 @@ int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* 
                  float scale, int causal, int dtype,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* ody_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * attention routine allocates through PyTorch.  Same arguments and results as ody_attn_fwd, bit
+ * for bit, without the workspace: the scratch of the bf16 head_dim-128 kernel (transposed image of
+ * V, block flags) lives in a buffer of ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES that the library itself
+ * holds on every GPU it runs on, for the life of the process.  The call allocates and frees
+ * nothing and synchronises nothing; a shape whose ody_attn_fwd_workspace_bytes exceeds the buffer
+ * (more than about 131000 key rows over all kv heads and batches) returns ODY_ERR_WORKSPACE.
+ * All calls on one GPU share that GPU's buffer: calls that may overlap there (different
+ * streams, different threads) race, so keep them on one stream or order them with events.  The
+ * first call on a device looks up the buffer's address; make that call outside graph capture.
+ */
+#define ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES ((32u << 20) + (64u << 10))
+int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                         int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                         int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                         int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                         int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                         int64_t so_b, int64_t so_l, int64_t so_h,
+                         float scale, int causal, int dtype, void* stream);
+
 /* Backward of the above (flash_attn's backward as run by autograd through
  * decoder/odysseus.py:256-263).  `out` and `lse` are the forward results -- or,
  * for a ring step, the FINAL merged out / lse, which is what makes the per-block

@@ -1,6 +1,12 @@
 // extern "C" entry points for attention.
 #include <cmath>
+#include <mutex>
 #include "attn_params.h"
+
+// Library-owned scratch of ody_attn_fwd_noalloc: one copy per GPU, held from the moment the code
+// object is loaded on that GPU until the process ends.  In host code this name is only a handle
+// for hipGetSymbolAddress; the device address is looked up once per device (scratch_of_device).
+static __device__ __align__(256) unsigned char scratch[ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -65,6 +71,50 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
   }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
   return ody_launch_attn_fwd_f32(p, D, st);
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (each GPU holds its own copy at its own address).
+int scratch_of_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  ODY_REQUIRE(e == hipSuccess && dev >= 0 && dev < kMaxDevices, ODY_ERR_LAUNCH,
+              "ody_attn_fwd_noalloc: no usable current device (%s)", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    ODY_REQUIRE(e == hipSuccess && ptr != nullptr, ODY_ERR_LAUNCH,
+                "ody_attn_fwd_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return ODY_OK;
+}
+}  // namespace
+
+extern "C" int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out, float* lse,
+                                    int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                                    int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                                    int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                                    int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                                    int64_t so_b, int64_t so_l, int64_t so_h,
+                                    float scale, int causal, int dtype, void* stream) {
+  int rc = check_common("ody_attn_fwd_noalloc", B, Lq, Lk, Hq, Hkv, D, dtype);
+  if (rc) return rc;
+  const size_t need = ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype);
+  ODY_REQUIRE(need <= (size_t)ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES, ODY_ERR_WORKSPACE,
+              "ody_attn_fwd_noalloc: this shape needs %zu bytes of scratch, the library-owned buffer holds %zu "
+              "(256 bytes per key row of every kv head: B*Hkv*Lk <= about 131000); use ody_attn_fwd with a "
+              "caller workspace", need, (size_t)ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (need > 0 && (rc = scratch_of_device(&ws))) return rc;
+  return ody_attn_fwd(q, k, v, out, lse, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h,
+                      so_b, so_l, so_h, scale, causal, dtype, ws, need, stream);
 }
 
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {

@@ -90,6 +90,25 @@ def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=No
     return out, lse
 
 
+def attn_fwd_noalloc(q, k, v, out, lse, causal: bool = True, scale: Optional[float] = None) -> None:
+    """attn_fwd into caller-owned `out` (B, Lq, Hq, D) and `lse` (B, Hq, Lq) fp32 without allocating
+    anything: the kernel's scratch is a buffer the library holds on the device.  Shapes beyond that
+    buffer (_lib.ATTN_FWD_NOALLOC_SCRATCH_BYTES) raise; calls that overlap on one device race."""
+    _need_gpu(q, k, v, out, lse)
+    B, Lq, Hq, D = q.shape
+    Lk, Hkv = k.shape[1], k.shape[2]
+    if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError(f"k {tuple(k.shape)} {k.dtype} / v {tuple(v.shape)} {v.dtype} do not match "
+                         f"q {tuple(q.shape)} {q.dtype}")
+    _same(q, "q", out=out)
+    if lse.dtype != torch.float32 or not lse.is_contiguous() or tuple(lse.shape) != (B, Hq, Lq):
+        raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    _lib.call("ody_attn_fwd_noalloc", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+              B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
+              scale, int(causal), _dt(q), _stream())
+
+
 def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
              dq=None, dk=None, dv=None, accumulate_dq: bool = False):
     """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step."""
