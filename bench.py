@@ -9,12 +9,17 @@ inputs, already resident in HBM).  `value` is the algorithmic TFLOP/s of that st
   roofline      the dominant kernel's algorithmic FLOP rate against the bf16 dense
                 MFMA peak, its duration measured with HIP events on the launch stream
   kernels       the same for every attention kernel of the step
+  step_ms       median / min / max of the K timed steps (HIP events around each step)
   mfma_sustained  what a loop of nothing but MFMAs sustains with constant and with random operands
-  layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs,
-                RoPE, RMSNorm, SwiGLU) and the resulting tokens/s
-  cpu_baseline  the CPU oracle timed on this host's cores on a bounded sample
+  configs       the other attention configurations (L = 131072; GQA 4:1 at L = 65536; the ring
+                step over 8 key blocks of 16384): ms, TFLOP/s, % of peak, forward / backward split
+  layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs with
+                torch.matmul on the same tensors as a same-box yardstick, RoPE, RMSNorm, SwiGLU)
+                and the resulting tokens/s as a sum of pieces
+  layer_end_to_end  the same share run through the modules and autograd
+  cpu_baseline  the CPU oracle timed on this host's cores: the whole step, and the layer's products once
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-layer]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-layer] [--no-configs]
 """
 from __future__ import annotations
 
@@ -54,6 +59,45 @@ def time_gpu(fn, iters, warmup):
     return (time.perf_counter() - t0) / iters
 
 
+def time_events(fn, iters, warmup):
+    """Per-call durations (ms) from HIP events recorded on the current stream around every call."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    torch.cuda.synchronize()
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) for a, b in evs)
+
+
+def spread(ms_sorted):
+    n = len(ms_sorted)
+    med = ms_sorted[n // 2] if n % 2 else 0.5 * (ms_sorted[n // 2 - 1] + ms_sorted[n // 2])
+    return {"median": round(med, 4), "min": round(ms_sorted[0], 4), "max": round(ms_sorted[-1], 4)}
+
+
+def kernel_ms(_lib, fn, iters, warmup):
+    """Average duration per call of the library's own kernels (HIP events on the launch stream),
+    summed over the kernels one call launches: (ms, {kernel: ms})."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    _lib.profile_collect()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    prof = _lib.profile_collect()
+    _lib.profile_enable(False)
+    per = {n: t / iters for n, (_, t, _) in prof.items()}
+    return sum(per.values()), per
+
+
 def measured_traffic():
     """HBM bytes per launch of the attention kernels at this workload, as measured with the
     FETCH_SIZE / WRITE_SIZE counters and recorded (as a JSON block) in the profile summary."""
@@ -88,21 +132,32 @@ def mfma_sustained(_lib, dev):
 
 
 def cpu_baseline():
-    """The oracle (plain PyTorch, fp32) on the host cores: causal attention fwd+bwd at
-    4 heads x 128, L = 16384 -- 1/4 of the FLOPs of one benchmark step (tens of core-seconds)."""
+    """The oracle (plain PyTorch, fp32) on the host cores: the whole benchmark step -- causal
+    attention fwd+bwd at 4 heads x 128, L = 32768 -- once (about 10 s on 16 cores), the three
+    products (forward, dgrad, wgrad) of the rank's four linears once, and the fp32 layer."""
     import torch
     sys.path.insert(0, str(ROOT / "oracle"))
     import odysseus_oracle as oracle
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     torch.set_num_threads(cores)
-    Ls = 16384
     g = torch.Generator().manual_seed(2000)
-    q, k, v, do = (torch.randn(1, Ls, H, D, generator=g) for _ in range(4))
+    q, k, v, do = (torch.randn(1, L, H, D, generator=g) for _ in range(4))
     t0 = time.perf_counter()
     o, lse = oracle.attention_fwd(q, k, v, causal=True)
     oracle.attention_bwd(q, k, v, o, lse, do, causal=True)
     dt = time.perf_counter() - t0
-    f, b = attn_flops(Ls, Ls, H, D)
+    del q, k, v, do, o, lse
+    f, b = attn_flops(L, L, H, D)
+    gemms = {}
+    for tag, (M, N, K) in (("qkv_proj", (L, (H + 2 * HKV) * D, D_MODEL)), ("o_proj", (L, D_MODEL, H * D)),
+                           ("gate_up_proj", (T_MLP, 2 * I_MLP, D_MODEL)), ("down_proj", (T_MLP, D_MODEL, I_MLP))):
+        x, w, dy = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g) * 0.02, torch.randn(M, N, generator=g)
+        t0 = time.perf_counter()
+        oracle.linear_fwd(x, w)
+        oracle.linear_bwd(x, w, dy)
+        tg = time.perf_counter() - t0
+        gemms[tag] = {"fwd_dgrad_wgrad_s": round(tg, 3), "tflops": round(6.0 * M * N * K / tg / 1e12, 3)}
+        del x, w, dy
     # the fp32 configuration as a whole on the same cores: one decoder layer forward + backward,
     # d=512, 8 heads x 64, i=1376, L=2048 (3 warm-up runs, 10 timed)
     Lc, dc, Hc, Dc, ic = 2048, 512, 8, 64, 1376
@@ -117,8 +172,8 @@ def cpu_baseline():
         oracle.decoder_layer_fwd_bwd(x, w, dy, Hc, Hc, Dc)
     layer_ms = (time.perf_counter() - t0) / 10 * 1e3
     return {"value": (f + b) / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"causal attention fwd+bwd, {H} heads x {D}, L={Ls} (1/4 of the step's FLOPs), fp32, "
-                      f"{dt:.2f} s wall",
+            "sample": f"the whole step once: causal attention fwd+bwd, {H} heads x {D}, L={L}, fp32, {dt:.2f} s wall",
+            "step_s": round(dt, 3), "linears_once": gemms,
             "fp32_layer_L2048_d512_ms": round(layer_ms, 2)}
 
 
@@ -129,6 +184,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=15)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-layer", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the L = 131072, GQA and ring configurations")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain device copy of the packed qkv buffer (100 MiB read + 100 MiB "
                          "written): the known-size kernel that calibrates the HBM byte counters of a "
@@ -184,6 +240,7 @@ def main():
     sec = (time.perf_counter() - t0) / a.steps
     prof = _lib.profile_collect()
     _lib.profile_enable(False)
+    step_spread = spread(time_events(step, a.steps, 0))   # a second pass: every step between its own pair of events
 
     f_fwd, f_bwd = attn_flops(L, L, H, D)
     # algorithmic FLOPs per launch: the backward's 5 tile products are S, dP, dV, dK (in the
@@ -224,7 +281,7 @@ def main():
                                "batch 1 (attention part of the 32768-token bf16 configuration)",
                    "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd,
                    "seeds": {"qkv": 2001, "dout": 2002}},
-        "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
+        "step_ms": step_spread, "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
         "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 1), "bwd_tflops": round(f_bwd / (bwd_ms * 1e-3) / 1e12, 1),
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "device": device,
@@ -238,14 +295,144 @@ def main():
     out["mfma_sustained"] = mfma_sustained(_lib, dev)
     # boxes differ by ~10 % in what they sustain at the power limit; this ratio does not
     out["value_over_mfma_sustained_random"] = round(value / out["mfma_sustained"]["random_operands_tflops"], 3)
-    if not a.no_layer:
-        out["layer"] = layer_share(_lib, ops, rn, dev, sec)
-        out["fp32"] = fp32_configuration(_lib, ops, dev)
     if a.power:
         out["power"] = power_under_load(_lib, ops, dev, step)
+    del qkv, q, k, v, do, dqkv
+    state.clear()
+    torch.cuda.empty_cache()
+    if not a.no_configs:
+        out["configs"] = other_configs(_lib, ops, rn, dev)
+    if not a.no_layer:
+        out["layer"] = layer_share(_lib, ops, rn, dev, sec)
+        out["layer_end_to_end"] = layer_end_to_end(_lib, rn, dev, out["layer"])
+        out["fp32"] = fp32_configuration(_lib, ops, dev)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
+
+
+FWD_KERNELS = ("attn_fwd_w8", "attn_fwd_mfma", "lse_merge")
+
+
+def other_configs(_lib, ops, rn, dev):
+    """The remaining attention configurations, each timed like the main step: a few whole steps between HIP
+    events, and the library's kernels by their own events for the forward / backward split."""
+    import torch
+    res = {}
+
+    def record(tag, step, flops_fwd, flops_bwd, iters, n_images_fwd, n_images, note):
+        ms = time_events(step, iters, 2)
+        _, per = kernel_ms(_lib, step, iters, 0)
+        img = per.get("attn_images", 0.0)
+        fwd = sum(t for n, t in per.items() if n in FWD_KERNELS) + img * n_images_fwd / max(n_images, 1)
+        bwd = sum(per.values()) - fwd
+        med = spread(ms)["median"]
+        tf = (flops_fwd + flops_bwd) / (med * 1e-3) / 1e12
+        res[tag] = {"workload": note, "step_ms": spread(ms), "tflops": round(tf, 1),
+                    "pct_of_bf16_peak": round(100 * tf / PEAK_BF16_TFLOPS, 2), "flops_per_step": flops_fwd + flops_bwd,
+                    "fwd_kernel_ms": round(fwd, 4), "bwd_kernel_ms": round(bwd, 4),
+                    "fwd_tflops": round(flops_fwd / (fwd * 1e-3) / 1e12, 1),
+                    "bwd_tflops": round(flops_bwd / (bwd * 1e-3) / 1e12, 1),
+                    "kernels_ms": {n: round(t, 4) for n, t in sorted(per.items())}}
+
+    def plain(tag, Lc, Hq, Hkv, seed, iters, note):
+        q, do = rn((1, Lc, Hq, D), seed), rn((1, Lc, Hq, D), seed + 3)
+        k, v = rn((1, Lc, Hkv, D), seed + 1), rn((1, Lc, Hkv, D), seed + 2)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+        def step():
+            o, lse = ops.attn_fwd(q, k, v, causal=True)
+            ops.attn_bwd(q, k, v, o, lse, do, causal=True, dq=dq, dk=dk, dv=dv)
+
+        f, b = attn_flops(Lc, Lc, Hq, D)
+        record(tag, step, f, b, iters, 1, 4, note)
+
+    plain("cfg3_L131072", 131072, 4, 4, 3000, 3, "causal attention fwd+bwd, 4 heads x 128, L=131072")
+    torch.cuda.empty_cache()
+    plain("cfg4_L65536_gqa4", 65536, 4, 1, 4000, 5, "causal attention fwd+bwd, 4 query heads on 1 kv head x 128, L=65536")
+    torch.cuda.empty_cache()
+
+    # the ring step: local queries against 8 key blocks, block 0 the causal diagonal, through autograd
+    Lq, NB = 16384, 8
+    q = rn((1, Lq, H, D), 5000).requires_grad_(True)
+    ks = [rn((1, Lq, H, D), 5001 + 2 * b).requires_grad_(True) for b in range(NB)]
+    vs = [rn((1, Lq, H, D), 5002 + 2 * b).requires_grad_(True) for b in range(NB)]
+    do = rn((1, Lq, H, D), 5100)
+
+    def ring_step():
+        for t in [q] + ks + vs:
+            t.grad = None
+        out, _ = ops.ring_blocks_attn(q, ks, vs, causal_block=0)
+        out.backward(do)
+
+    f_full, b_full = attn_flops(Lq, Lq, H, D, causal=False)
+    f_diag, b_diag = attn_flops(Lq, Lq, H, D, causal=True)
+    record("cfg5_ring_8x16384", ring_step, 7 * f_full + f_diag, 7 * b_full + b_diag, 5, NB, 4 * NB,
+           "ring step through autograd: 16384 queries x 4 heads x 128 against 8 key blocks of 16384 "
+           "(block 0 causal), LSE merge after each, backward over all 8")
+    return res
+
+
+def layer_end_to_end(_lib, rn, dev, pieces):
+    """One rank's share of a layer run through the modules and autograd instead of summed from separately
+    timed pieces: LlamaFlashAttention2TPSP on the gathered 32768 tokens (packed QKV projection, RoPE, attention,
+    output projection; forward + backward), and on the 4096-token shard RMSNorm -> LlamaMLPZeRO plus the other
+    RMSNorm and both residual adds.  Host overhead, workspace handling and autograd bookkeeping are inside."""
+    import types
+    import torch
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP, LlamaMLPZeRO, LlamaRMSNorm
+    from odysseus_transformer_amd.utils import globals as arena
+    cfg = types.SimpleNamespace(hidden_size=D_MODEL, num_attention_heads=H, num_key_value_heads=HKV, head_dim=D,
+                                intermediate_size=I_MLP, hidden_act="silu", attention_dropout=0.0, rms_norm_eps=1e-6,
+                                rope_theta=10000.0, max_position_embeddings=1 << 20, pretraining_tp=1,
+                                num_hidden_layers=1)
+    dt = torch.bfloat16
+    if arena._Arena.instance is None:
+        arena._set_global_memory_buffer(dev)
+    attn = LlamaFlashAttention2TPSP(cfg, 0).to(dt).to(dev)
+    mlp = LlamaMLPZeRO(cfg).to(dt).to(dev)
+    n1, n2 = LlamaRMSNorm(D_MODEL).to(dt).to(dev), LlamaRMSNorm(D_MODEL).to(dt).to(dev)
+    with torch.no_grad():
+        for i, w in enumerate(list(attn.parameters()) + list(mlp.parameters())):
+            w.copy_(rn(tuple(w.shape), 9000 + i, 0.02))
+    x_full = rn((1, L, D_MODEL), 9100).requires_grad_(True)     # the gathered, normalised activation
+    dy_full = rn((1, L, D_MODEL), 9101)
+    x_loc = rn((1, T_MLP, D_MODEL), 9102).requires_grad_(True)
+    dy_loc = rn((1, T_MLP, D_MODEL), 9103)
+    pos = torch.arange(L, device=dev)[None]
+    params = list(attn.parameters()) + list(mlp.parameters()) + list(n1.parameters()) + list(n2.parameters())
+
+    def attn_part():
+        attn(x_full, position_ids=pos)[0].backward(dy_full)
+
+    from odysseus_transformer_amd import ops as _ops
+
+    def shard_part():
+        a = n1(x_loc)                      # the norm in front of the attention block (its output is what gets gathered)
+        h = x_loc + a                      # stands in for the residual add after the reduce-scatter of the attention block
+        # second norm, SwiGLU MLP and the second residual add with the elementwise steps in the products' epilogues
+        n, skip = _ops.rmsnorm_fork(h, n2.weight, n2.variance_epsilon)
+        mlp(n, residual=skip).backward(dy_loc)
+
+    def whole():
+        for t in params + [x_full, x_loc]:
+            t.grad = None
+        attn_part()
+        shard_part()
+
+    ms = time_events(whole, 10, 3)
+    ms_attn = time_events(lambda: ([setattr(t, "grad", None) for t in params + [x_full]], attn_part()), 10, 1)
+    ms_shard = time_events(lambda: ([setattr(t, "grad", None) for t in params + [x_loc]], shard_part()), 10, 1)
+    med = spread(ms)["median"]
+    arena._destroy_global_memory_buffer()
+    return {"workload": "LlamaFlashAttention2TPSP (32768 gathered tokens, 4 x 128 heads) + RMSNorm / LlamaMLPZeRO / "
+                        "residual adds on the 4096-token shard, forward + backward through autograd",
+            "ms": spread(ms), "attention_block_ms": spread(ms_attn), "shard_part_ms": spread(ms_shard),
+            "layer_tokens_per_s_per_gpu": round(T_MLP / (med * 1e-3), 1),
+            "sum_of_pieces_tokens_per_s_per_gpu": pieces["layer_tokens_per_s_per_gpu"],
+            "scratch": "attention, split-K and norm workspaces drawn from the GlobalMemoryBuffer arena",
+            "fusions": "SwiGLU forward / backward and the MLP's residual add run in GEMM epilogues, the gradient sum at the "
+                       "fork of the residual stream inside the RMSNorm backward"}
 
 
 def layer_share(_lib, ops, rn, dev, attn_sec):
@@ -256,16 +443,29 @@ def layer_share(_lib, ops, rn, dev, attn_sec):
     res = {}
 
     def gemm3(tag, M, N, K):
+        """The three products of one linear, 20 calls each: the library's kernels by their own HIP events, and
+        torch.matmul on the same tensors by events on the same stream as a same-box yardstick (measurement
+        only: it is not on any product path)."""
         x, w, dy = rn((M, K), 1), rn((N, K), 2, 0.02), rn((M, N), 3)
-        tf = time_gpu(lambda: ops.gemm(ops.GEMM_NT, x, w), 5, 2)
-        td = time_gpu(lambda: ops.gemm(ops.GEMM_NN, dy, w), 5, 2)
-        tw = time_gpu(lambda: ops.gemm(ops.GEMM_TN, dy, x), 5, 2)
         fl = 2.0 * M * N * K
-        res[tag] = {"M": M, "N": N, "K": K, "fwd_ms": round(tf * 1e3, 3), "dgrad_ms": round(td * 1e3, 3),
-                    "wgrad_ms": round(tw * 1e3, 3),
-                    "tflops": [round(fl / t / 1e12, 1) for t in (tf, td, tw)]}
+        mine, yard, kern = [], [], {}
+        for name, ours, theirs in (("fwd", lambda: ops.gemm(ops.GEMM_NT, x, w), lambda: torch.matmul(x, w.t())),
+                                   ("dgrad", lambda: ops.gemm(ops.GEMM_NN, dy, w), lambda: torch.matmul(dy, w)),
+                                   ("wgrad", lambda: ops.gemm(ops.GEMM_TN, dy, x), lambda: torch.matmul(dy.t(), x))):
+            t, per = kernel_ms(_lib, ours, 20, 3)
+            mine.append(t * 1e-3)
+            kern[name] = sorted(per)
+            yard.append(spread(time_events(theirs, 20, 3))["median"] * 1e-3)
+        res[tag] = {"M": M, "N": N, "K": K, "fwd_ms": round(mine[0] * 1e3, 4), "dgrad_ms": round(mine[1] * 1e3, 4),
+                    "wgrad_ms": round(mine[2] * 1e3, 4), "tflops": [round(fl / t / 1e12, 1) for t in mine],
+                    "frac_of_bf16_peak": [round(fl / t / 1e12 / PEAK_BF16_TFLOPS, 3) for t in mine],
+                    "kernels": kern,
+                    "yardstick": {"what": "torch.matmul on the same tensors (hipBLASLt), median of 20 by HIP events",
+                                  "ms": [round(t * 1e3, 4) for t in yard],
+                                  "tflops": [round(fl / t / 1e12, 1) for t in yard],
+                                  "ours_over_yardstick": [round(ty / tm, 3) for tm, ty in zip(mine, yard)]}}
         del x, w, dy
-        return tf + td + tw
+        return sum(mine)
 
     def membound(tag, fn, nbytes):
         # wall clock per call (what the layer total uses; for kernels this short it includes the host's

@@ -177,6 +177,35 @@ int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias,
              int M, int N, int K, int64_t lda, int64_t ldb, int64_t ldc,
              int accumulate, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- linears fused with their elementwise neighbour -----------------------------
+ * The same products as ody_gemm's NT / NN with the operation that follows them in the layer done in the
+ * product's epilogue, so that the intermediate never makes a round trip through HBM.  Row-major, leading
+ * dimensions in elements.  bf16 shapes made of whole 256 x 256 tiles with K a multiple of 64 and 16-byte
+ * aligned rows take one fused kernel; everything else (fp32, ragged or small shapes) runs as the product
+ * followed by the stand-alone kernel, with the same result.
+ *
+ * ody_linear_residual     y (M, N) = x (M, K) W (N, K)^T + residual (M, N): the output projection and the
+ *                         down projection together with the decoder layer's residual add
+ *                         (utils/linear_tpsp.py:588 / utils/linear_zero3.py:44, then decoder/ring.py:80,86).
+ *                         The sum is formed in fp32 and rounded once.  y may be the residual buffer itself only
+ *                         when the shape takes the unfused path; pass distinct buffers.
+ * ody_linear_swiglu       gate_up (T, 2 I) = x (T, K) Wgu (2 I, K)^T and h (T, I) = silu(gate) * up
+ *                         (decoder/odysseus.py:293-295); gate_up is kept because the backward needs it.
+ * ody_linear_dgrad_swiglu d_gate_up (T, 2 I) = SwiGLU backward of (gate_up, dh) with dh = dy (T, K) Wd (K, I):
+ *                         the input gradient of the down projection (utils/linear_zero3.py:68) feeding the
+ *                         backward of decoder/odysseus.py:295; dh itself is never stored.  workspace:
+ *                         ody_linear_dgrad_swiglu_workspace_bytes(...) bytes (0 when the fused kernel applies;
+ *                         otherwise room for dh), 16-byte aligned.
+ */
+int ody_linear_residual(const void* x, const void* w, const void* residual, void* y, int M, int N, int K,
+                        int64_t ldx, int64_t ldw, int64_t ld_res, int64_t ldy, int dtype, void* stream);
+int ody_linear_swiglu(const void* x, const void* w_gate_up, void* gate_up, void* h, int T, int I, int K,
+                      int64_t ldx, int64_t ldw, int64_t ld_gu, int64_t ld_h, int dtype, void* stream);
+size_t ody_linear_dgrad_swiglu_workspace_bytes(int T, int I, int K, int dtype);
+int ody_linear_dgrad_swiglu(const void* dy, const void* w_down, const void* gate_up, void* d_gate_up, int T, int I,
+                            int K, int64_t ld_dy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- SwiGLU -------------------------------------------------------------
  * decoder/odysseus.py:293-295: a1, a3 = gate_up.chunk(2, -1); h = silu(a1) * a3.
  * gate_up (T, 2*I) row stride ld_gu; h (T, I) row stride ld_h.
@@ -193,12 +222,16 @@ int ody_swiglu_bwd(const void* gate_up, const void* dh, void* d_gate_up, int T, 
  * contiguous; rstd (T) fp32 is written by fwd and read by bwd.
  * bwd: dx (T, d); dw_partial (n_partial, d) fp32 partial column sums, where
  * n_partial = ody_rmsnorm_bwd_partials(T); the caller (or ody_rmsnorm_bwd with
- * dw != NULL) reduces them: dw (d) of `dtype`.
+ * dw != NULL) reduces them: dw (d) of `dtype`.  dx_add (T, d) of `dtype` or NULL is
+ * added to dx in fp32 before the one rounding: the gradient that reaches the
+ * norm's input over the residual connection (decoder/ring.py:80,86), so that the
+ * sum of the two branches costs no pass of its own.  d at most 8192 (bf16) /
+ * 4096 (fp32): larger rows return ODY_ERR_UNSUPPORTED.
  */
 int ody_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int T, int d, float eps,
                     int dtype, void* stream);
 int ody_rmsnorm_bwd_partials(int T);
-int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
+int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, const void* dx_add, void* dx,
                     float* dw_partial, void* dw, int T, int d, int dtype, void* stream);
 
 /* ---- RoPE ---------------------------------------------------------------

@@ -33,11 +33,15 @@ SIGNATURES = {
     "ody_lse_merge": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i, _p]),
     "ody_gemm_workspace_bytes": (_sz, [_i] * 5),
     "ody_gemm": (_i, [_i] + [_p] * 4 + [_i] * 3 + [_i64] * 3 + [_i, _i, _p, _sz, _p]),
+    "ody_linear_residual": (_i, [_p] * 4 + [_i] * 3 + [_i64] * 4 + [_i, _p]),
+    "ody_linear_swiglu": (_i, [_p] * 4 + [_i] * 3 + [_i64] * 4 + [_i, _p]),
+    "ody_linear_dgrad_swiglu_workspace_bytes": (_sz, [_i] * 4),
+    "ody_linear_dgrad_swiglu": (_i, [_p] * 4 + [_i] * 3 + [_i64] * 4 + [_i, _p, _sz, _p]),
     "ody_swiglu_fwd": (_i, [_p, _p, _i, _i, _i64, _i64, _i, _p]),
     "ody_swiglu_bwd": (_i, [_p, _p, _p, _i, _i, _i64, _i64, _i64, _i, _p]),
     "ody_rmsnorm_fwd": (_i, [_p] * 4 + [_i, _i, _f, _i, _p]),
     "ody_rmsnorm_bwd_partials": (_i, [_i]),
-    "ody_rmsnorm_bwd": (_i, [_p] * 7 + [_i, _i, _i, _p]),
+    "ody_rmsnorm_bwd": (_i, [_p] * 8 + [_i, _i, _i, _p]),
     "ody_cross_entropy_fwd": (_i, [_p] * 5 + [_i, _i, _i64, _i64, _i, _p]),
     "ody_cross_entropy_bwd": (_i, [_p] * 6 + [_i, _i, _i64, _i64, _i, _p]),
     "ody_rope": (_i, [_p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _f, _i, _i, _p]),

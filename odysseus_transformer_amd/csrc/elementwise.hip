@@ -98,7 +98,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const float* __restrict__ rstd, const T* __restrict__ dy,
                                                           T* __restrict__ dx, float* __restrict__ dw_partial,
-                                                          int Trows, int d, int rows_per_block) {
+                                                          int Trows, int d, int rows_per_block,
+                                                          const T* __restrict__ dx_add) {
   constexpr int N = VecIO<T>::N, MAXK = RMS_BWD_MAXK;
   __shared__ float red[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -141,9 +142,12 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     for (int k = 0; k < MAXK; k++) {
       const int vi = tid + 256 * k;
       if (vi < nvec) {
-        float o[N];
+        float o[N], add[N];
 #pragma unroll
-        for (int e = 0; e < N; e++) o[e] = rs * (gv[k][e] - xh[k][e] * c);
+        for (int e = 0; e < N; e++) add[e] = 0.f;
+        if (dx_add) VecIO<T>::load(dx_add + (int64_t)row * d + vi * N, add);   // gradient arriving over the residual path
+#pragma unroll
+        for (int e = 0; e < N; e++) o[e] = add[e] + rs * (gv[k][e] - xh[k][e] * c);
         VecIO<T>::store(dx + (int64_t)row * d + vi * N, o);
       }
     }
@@ -345,24 +349,26 @@ extern "C" int ody_rmsnorm_fwd(const void* x, const void* w, void* y, float* rst
 
 extern "C" int ody_rmsnorm_bwd_partials(int T) { return T <= 0 ? 0 : (T < 512 ? T : 512); }
 
-extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
-                               float* dw_partial, void* dw, int T, int d, int dtype, void* stream) {
+extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, const void* dx_add,
+                               void* dx, float* dw_partial, void* dw, int T, int d, int dtype, void* stream) {
   ODY_REQUIRE(x && w && rstd && dy && dx && dw_partial, ODY_ERR_NULL, "ody_rmsnorm_bwd: NULL pointer");
   ODY_REQUIRE(T > 0 && d > 0, ODY_ERR_BAD_SHAPE, "ody_rmsnorm_bwd: T=%d d=%d", T, d);
   const int n = dtype == ODY_BF16 ? 8 : 4;
   ODY_REQUIRE(d % n == 0 && d <= 256 * n * RMS_BWD_MAXK, ODY_ERR_UNSUPPORTED,
               "ody_rmsnorm_bwd: d=%d must be a multiple of %d and at most %d", d, n, 256 * n * RMS_BWD_MAXK);
-  ODY_REQUIRE(ody_aligned16(x) && ody_aligned16(w) && ody_aligned16(dy) && ody_aligned16(dx), ODY_ERR_MISALIGNED,
-              "ody_rmsnorm_bwd: pointers must be 16-byte aligned");
+  ODY_REQUIRE(ody_aligned16(x) && ody_aligned16(w) && ody_aligned16(dy) && ody_aligned16(dx) && ody_aligned16(dx_add),
+              ODY_ERR_MISALIGNED, "ody_rmsnorm_bwd: pointers must be 16-byte aligned");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int nparts = ody_rmsnorm_bwd_partials(T);
   const int rpb = (T + nparts - 1) / nparts;
   const int nblocks = (T + rpb - 1) / rpb;  // <= nparts; rows of dw_partial beyond nblocks are not written
   ODY_BY_DTYPE(dtype,
                ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<bf16>, dim3(nblocks), dim3(256), 0, (const bf16*)x,
-                                  (const bf16*)w, rstd, (const bf16*)dy, (bf16*)dx, dw_partial, T, d, rpb),
+                                  (const bf16*)w, rstd, (const bf16*)dy, (bf16*)dx, dw_partial, T, d, rpb,
+                                  (const bf16*)dx_add),
                ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<float>, dim3(nblocks), dim3(256), 0, (const float*)x,
-                                  (const float*)w, rstd, (const float*)dy, (float*)dx, dw_partial, T, d, rpb));
+                                  (const float*)w, rstd, (const float*)dy, (float*)dx, dw_partial, T, d, rpb,
+                                  (const float*)dx_add));
   int rc = ody_check_launch("rmsnorm_bwd");
   if (rc || !dw) return rc;
   ODY_BY_DTYPE(dtype,

@@ -76,16 +76,35 @@ struct OperandTile {
 // k-step.
 #define GEMM_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// What the fast kernel's epilogue does besides rounding and storing the tile.
+//   EPI_RESIDUAL    C = A B + R                      (R = aux, row pitch ld_aux; one rounding, after the add)
+//   EPI_SWIGLU_FWD  NT only.  B is the packed (2 I, K) gate_up weight.  A 256-column tile holds 128 gate columns
+//                   and the 128 matching up columns, interleaved in blocks of 32 (block c of the tile: gate if c is
+//                   even, up if odd, columns j0 + 32 (c / 2) ...), so that a lane owns gate and up of the same
+//                   (token, j).  Writes gate_up to C in its usual [gate | up] layout and h = silu(gate) * up to out2,
+//                   computed from the rounded gate / up values exactly as the stand-alone SwiGLU kernel would.
+//   EPI_SWIGLU_BWD  the tile is dh = dy Wd (N = I); with gate_up = aux the epilogue writes d_gate_up to C (pitch
+//                   ldc, 2 I columns) as the stand-alone SwiGLU backward would from the rounded dh.
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU_FWD = 2, EPI_SWIGLU_BWD = 3 };
+struct GemmEpi {
+  const bf16* aux;
+  bf16* out2;
+  int64_t ld_aux, ld_out2;
+  int I;
+};
+
 //
 // SPLITK: blockIdx.y selects one of gridDim.y ranges of K slabs; the block writes its fp32 partial tile to
 // part[blockIdx.y][M][N] and gemm_splitk_sum_kernel adds the ranges up (bias, C += and the rounding happen
 // there).  For products with a long K and few output tiles (weight gradients) this is what fills the chip.
-template <int WM, int WN, bool A_KC, bool B_KC, bool SPLITK>
+template <int WM, int WN, bool A_KC, bool B_KC, bool SPLITK, int EPI = EPI_NONE>
 __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
                                                              bf16* __restrict__ C, const bf16* __restrict__ bias,
                                                              int M, int N, int K, int64_t lda, int64_t ldb,
                                                              int64_t ldc, int accumulate, int tiles_m, int tiles_n,
-                                                             float* __restrict__ part) {
+                                                             float* __restrict__ part, GemmEpi ep) {
+  static_assert(EPI == EPI_NONE || (!SPLITK && WM == 4 && WN == 4), "fused epilogues: 256 x 256 tiles, one pass over K");
+  static_assert(EPI != EPI_SWIGLU_FWD || (A_KC && B_KC), "the SwiGLU forward epilogue belongs to the NT product");
   constexpr int TM = 64 * WM, TN = 64 * WN;
   typedef OperandTile<TM, A_KC> TA;
   typedef OperandTile<TN, B_KC> TB;
@@ -135,7 +154,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     nk = max(0, min(nk - kt0, per));
   }
   const bf16* Abase = (A_KC ? A + (int64_t)m0 * lda : A + m0) + (int64_t)kt0 * a_slab;   // first element of the first slab
-  const bf16* Bbase = (B_KC ? B + (int64_t)n0 * ldb : B + n0) + (int64_t)kt0 * b_slab;
+  // EPI_SWIGLU_FWD: tile tn covers j in [128 tn, 128 tn + 128); chunk j of a thread lies in the tile's 32-row block j
+  const bf16* Bbase = (EPI == EPI_SWIGLU_FWD ? B + (int64_t)(n0 / 2) * ldb : (B_KC ? B + (int64_t)n0 * ldb : B + n0)) +
+                      (int64_t)kt0 * b_slab;
+  const int64_t b_up = (int64_t)ep.I * ldb;   // from a gate row to its up row
 
   f32x16 acc[WM][WN];
 #pragma unroll
@@ -150,7 +172,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     ra[j] = *reinterpret_cast<const bf16x8*>(Abase + (int64_t)kt * a_slab + j * a_step + a_off0);
   };
   auto gload_b = [&](int kt, int j) {
-    rb[j] = *reinterpret_cast<const bf16x8*>(Bbase + (int64_t)kt * b_slab + j * b_step + b_off0);
+    const int64_t rows = EPI == EPI_SWIGLU_FWD ? (j & 1) * b_up + (j >> 1) * b_step : j * b_step;
+    rb[j] = *reinterpret_cast<const bf16x8*>(Bbase + (int64_t)kt * b_slab + rows + b_off0);
   };
   auto sstore_a = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(As + buf * TA::ELEMS + a_lds0 + j * a_lstep) = ra[j]; };
   auto sstore_b = [&](int buf, int j) { *reinterpret_cast<bf16x8*>(Bs + buf * TB::ELEMS + b_lds0 + j * b_lstep) = rb[j]; };
@@ -243,6 +266,123 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
         const int row = pass * RPP + lane / CPR, c = lane % CPR;
         const f32x4 v = *reinterpret_cast<const f32x4*>(band + row * EPF + 4 * c);
         *reinterpret_cast<f32x4*>(dst0 + (int64_t)(32 * (wm * WM + a) + row) * N + 4 * c) = v;
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == EPI_RESIDUAL) {
+    // fp32 bands, so that the residual is added before the one rounding; 16-byte pieces of whole rows of R and C
+    constexpr int EPF = 32 * WN + 4;
+    float* band = reinterpret_cast<float*>(smem_raw) + wave * 32 * EPF;
+    static_assert(4 * 32 * EPF * 2 <= 2 * (TA::ELEMS + TB::ELEMS), "the fp32 bands fit in the operand buffers");
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          f32x4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          *reinterpret_cast<f32x4*>(band + i * EPF + 32 * b + 8 * q + 4 * g) = v;
+        }
+      constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const f32x4 v0 = *reinterpret_cast<const f32x4*>(band + row * EPF + 8 * c);
+        const f32x4 v1 = *reinterpret_cast<const f32x4*>(band + row * EPF + 8 * c + 4);
+        const int m = m0 + 32 * (wm * WM + a) + row, n = n0 + 32 * wn * WN + 8 * c;
+        const bf16x8 r = *reinterpret_cast<const bf16x8*>(ep.aux + (int64_t)m * ep.ld_aux + n);
+        bf16x8 w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = (bf16)(v0[e] + (float)r[e]), w[4 + e] = (bf16)(v1[e] + (float)r[4 + e]);
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + n) = w;
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == EPI_SWIGLU_FWD) {
+    constexpr int EP = 32 * WN + 8, EPH = 16 * WN + 8;
+    bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;
+    const int j0 = n0 / 2;   // first j of the tile
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+      bf16x4 gu[WN][4];
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) gu[b][q][e] = (bf16)acc[a][b][4 * q + e];
+          *reinterpret_cast<bf16x4*>(band + i * EP + 32 * b + 8 * q + 4 * g) = gu[b][q];
+        }
+      constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const bf16x8 w = *reinterpret_cast<const bf16x8*>(band + row * EP + 8 * c);
+        const int m = m0 + 32 * (wm * WM + a) + row, blk = wn * WN + c / 4;   // 32-column block of the tile
+        const int col = (blk & 1) * ep.I + j0 + 32 * (blk >> 1) + 8 * (c % 4);
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + col) = w;
+      }
+      // h from the rounded values; blocks 2 p (gate) and 2 p + 1 (up) of this wavefront pair up
+#pragma unroll
+      for (int pr = 0; pr < WN / 2; pr++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          bf16x4 hv;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float a1 = (float)gu[2 * pr][q][e], a3 = (float)gu[2 * pr + 1][q][e];
+            hv[e] = (bf16)(a1 / (1.f + __expf(-a1)) * a3);
+          }
+          *reinterpret_cast<bf16x4*>(band + i * EPH + 32 * pr + 8 * q + 4 * g) = hv;
+        }
+      constexpr int CPRH = 16 * WN / 8, RPPH = 64 / CPRH;
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPPH; pass++) {
+        const int row = pass * RPPH + lane / CPRH, c = lane % CPRH;
+        const bf16x8 w = *reinterpret_cast<const bf16x8*>(band + row * EPH + 8 * c);
+        const int m = m0 + 32 * (wm * WM + a) + row;
+        const int col = j0 + 32 * (wn * (WN / 2) + c / 4) + 8 * (c % 4);
+        *reinterpret_cast<bf16x8*>(ep.out2 + (int64_t)m * ep.ld_out2 + col) = w;
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == EPI_SWIGLU_BWD) {
+    constexpr int EP = 32 * WN + 8;
+    bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          bf16x4 w;
+#pragma unroll
+          for (int e = 0; e < 4; e++) w[e] = (bf16)acc[a][b][4 * q + e];
+          *reinterpret_cast<bf16x4*>(band + i * EP + 32 * b + 8 * q + 4 * g) = w;
+        }
+      constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const bf16x8 dh = *reinterpret_cast<const bf16x8*>(band + row * EP + 8 * c);
+        const int m = m0 + 32 * (wm * WM + a) + row, j = n0 + 32 * wn * WN + 8 * c;
+        const bf16x8 gt = *reinterpret_cast<const bf16x8*>(ep.aux + (int64_t)m * ep.ld_aux + j);
+        const bf16x8 up = *reinterpret_cast<const bf16x8*>(ep.aux + (int64_t)m * ep.ld_aux + ep.I + j);
+        bf16x8 d1, d3;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float a1 = (float)gt[e], a3 = (float)up[e], gg = (float)dh[e];
+          const float sig = 1.f / (1.f + __expf(-a1));
+          d1[e] = (bf16)(gg * a3 * sig * (1.f + a1 * (1.f - sig)));
+          d3[e] = (bf16)(gg * a1 * sig);
+        }
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + j) = d1;
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + ep.I + j) = d3;
       }
     }
     return;
@@ -479,7 +619,7 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
                         (int64_t)BK * ldb < (1ll << 31);
   if (interior && splits > 1) {
     ODY_LAUNCH(name, st, fastk, dim3(tiles_m * tiles_n, splits), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
-               accumulate, tiles_m, tiles_n, part);
+               accumulate, tiles_m, tiles_n, part, GemmEpi{});
     int rc = ody_check_launch("gemm_bf16");
     if (rc) return rc;
     const int64_t n4 = (int64_t)M * (N / 4);
@@ -489,7 +629,7 @@ int launch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M, 
   }
   if (interior) {
     ODY_LAUNCH(name, st, fast, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
-               accumulate, tiles_m, tiles_n, nullptr);
+               accumulate, tiles_m, tiles_n, nullptr, GemmEpi{});
     return ody_check_launch("gemm_bf16");
   }
   ODY_LAUNCH(name, st, kern, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, bias, M, N, K, lda, ldb, ldc,
@@ -511,6 +651,24 @@ int dispatch_bf16(const bf16* A, const bf16* B, bf16* C, const bf16* bias, int M
   if (big_tiles >= 192)
     return launch_bf16<4, 4, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, nullptr, 1, st);
   return launch_bf16<2, 2, A_KC, B_KC>(A, B, C, bias, M, N, K, lda, ldb, ldc, accumulate, nullptr, 1, st);
+}
+
+// Whether a product of these sizes can take the 256 x 256 fast kernel in one pass over K (what the fused epilogues need).
+bool fused_shape_ok(int M, int N, int K, int64_t lda, int64_t ldb) {
+  return M % 256 == 0 && N % 256 == 0 && K % BK == 0 && 256 * lda < (1ll << 31) && 256 * ldb < (1ll << 31) &&
+         BK * lda < (1ll << 31) && BK * ldb < (1ll << 31);
+}
+
+template <bool B_KC, int EPI>
+int launch_fused(const char* name, const bf16* A, const bf16* B, bf16* C, int M, int N, int K, int64_t lda, int64_t ldb,
+                 int64_t ldc, const GemmEpi& ep, hipStream_t st) {
+  constexpr size_t smem = 2 * sizeof(bf16) * (OperandTile<256, true>::ELEMS + OperandTile<256, B_KC>::ELEMS);
+  auto kern = &gemm_bf16_fast_kernel<4, 4, true, B_KC, false, EPI>;
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, name)) return rc;
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  ODY_LAUNCH(name, st, kern, dim3(tiles_m * tiles_n), dim3(256), smem, A, B, C, static_cast<const bf16*>(nullptr), M, N,
+             K, lda, ldb, ldc, 0, tiles_m, tiles_n, static_cast<float*>(nullptr), ep);
+  return ody_check_launch(name);
 }
 
 // One bf16 product.  A ragged M or N is cut into a main part of whole tiles, which takes the fast
@@ -764,4 +922,97 @@ extern "C" int ody_gemm(int op, const void* A, const void* B, void* C, const voi
               "(M=%d N=%d K=%d op=%d)", M, N, K, op);
   return gemm_bf16(op, (const bf16*)A, (const bf16*)B, (bf16*)C, (const bf16*)bias, M, N, K, lda, ldb, ldc, accumulate,
                    workspace, workspace_bytes, st);
+}
+
+// ---------------------------------------------------------------------------
+// Linears with the neighbouring elementwise operation in their epilogue
+// ---------------------------------------------------------------------------
+namespace {
+int check_lin(const char* who, const void* a, const void* b, const void* c, int M, int N, int K, int dtype) {
+  ODY_REQUIRE(a && b && c, ODY_ERR_NULL, "%s: NULL pointer", who);
+  ODY_REQUIRE(M > 0 && N > 0 && K > 0, ODY_ERR_BAD_SHAPE, "%s: M=%d N=%d K=%d", who, M, N, K);
+  ODY_REQUIRE(dtype == ODY_BF16 || dtype == ODY_F32, ODY_ERR_UNSUPPORTED, "%s: dtype %d unknown", who, dtype);
+  return ODY_OK;
+}
+bool vec16(const void* p, int64_t ld) { return ody_aligned16(p) && ld % 8 == 0; }
+}  // namespace
+
+extern "C" int ody_linear_residual(const void* x, const void* w, const void* residual, void* y, int M, int N, int K,
+                                   int64_t ldx, int64_t ldw, int64_t ld_res, int64_t ldy, int dtype, void* stream) {
+  int rc = check_lin("ody_linear_residual", x, w, y, M, N, K, dtype);
+  if (rc) return rc;
+  ODY_REQUIRE(residual != nullptr, ODY_ERR_NULL, "ody_linear_residual: residual is NULL");
+  ODY_REQUIRE(ldx >= K && ldw >= K && ld_res >= N && ldy >= N, ODY_ERR_BAD_SHAPE,
+              "ody_linear_residual: leading dimension smaller than the row length");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && fused_shape_ok(M, N, K, ldx, ldw) && vec16(x, ldx) && vec16(w, ldw) && vec16(residual, ld_res) &&
+      vec16(y, ldy) && (int64_t)((M + 255) / 256) * ((N + 255) / 256) >= 128) {
+    GemmEpi ep{static_cast<const bf16*>(residual), nullptr, ld_res, 0, 0};
+    return launch_fused<true, EPI_RESIDUAL>("gemm_bf16_nt_residual", static_cast<const bf16*>(x), static_cast<const bf16*>(w),
+                                            static_cast<bf16*>(y), M, N, K, ldx, ldw, ldy, ep, st);
+  }
+  // any other shape or type: y = residual, then y += x W^T (added in fp32 before the one rounding, as above)
+  if (y != residual) {
+    const size_t es = dtype == ODY_BF16 ? 2 : 4;
+    hipError_t e = hipMemcpy2DAsync(y, (size_t)ldy * es, residual, (size_t)ld_res * es, (size_t)N * es, (size_t)M,
+                                    hipMemcpyDeviceToDevice, st);
+    ODY_REQUIRE(e == hipSuccess, ODY_ERR_LAUNCH, "ody_linear_residual: copy of the residual failed: %s", hipGetErrorString(e));
+  }
+  return ody_gemm(ODY_GEMM_NT, x, w, y, nullptr, M, N, K, ldx, ldw, ldy, 1, dtype, nullptr, 0, stream);
+}
+
+extern "C" int ody_swiglu_fwd(const void* gate_up, void* h, int T, int I, int64_t ld_gu, int64_t ld_h, int dtype,
+                              void* stream);
+extern "C" int ody_swiglu_bwd(const void* gate_up, const void* dh, void* d_gate_up, int T, int I, int64_t ld_gu,
+                              int64_t ld_dh, int64_t ld_dgu, int dtype, void* stream);
+
+extern "C" int ody_linear_swiglu(const void* x, const void* w_gate_up, void* gate_up, void* h, int T, int I, int K,
+                                 int64_t ldx, int64_t ldw, int64_t ld_gu, int64_t ld_h, int dtype, void* stream) {
+  int rc = check_lin("ody_linear_swiglu", x, w_gate_up, gate_up, T, I, K, dtype);
+  if (rc) return rc;
+  ODY_REQUIRE(h != nullptr, ODY_ERR_NULL, "ody_linear_swiglu: h is NULL");
+  ODY_REQUIRE(ldx >= K && ldw >= K && ld_gu >= 2 * (int64_t)I && ld_h >= I, ODY_ERR_BAD_SHAPE,
+              "ody_linear_swiglu: leading dimension smaller than the row length");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && I % 128 == 0 && fused_shape_ok(T, 2 * I, K, ldx, ldw) && (int64_t)I * ldw < (1ll << 40) &&
+      vec16(x, ldx) && vec16(w_gate_up, ldw) && vec16(gate_up, ld_gu) && vec16(h, ld_h)) {
+    GemmEpi ep{nullptr, static_cast<bf16*>(h), 0, ld_h, I};
+    return launch_fused<true, EPI_SWIGLU_FWD>("gemm_bf16_nt_swiglu", static_cast<const bf16*>(x),
+                                              static_cast<const bf16*>(w_gate_up), static_cast<bf16*>(gate_up), T, 2 * I, K,
+                                              ldx, ldw, ld_gu, ep, st);
+  }
+  rc = ody_gemm(ODY_GEMM_NT, x, w_gate_up, gate_up, nullptr, T, 2 * I, K, ldx, ldw, ld_gu, 0, dtype, nullptr, 0, stream);
+  if (rc) return rc;
+  return ody_swiglu_fwd(gate_up, h, T, I, ld_gu, ld_h, dtype, stream);
+}
+
+extern "C" size_t ody_linear_dgrad_swiglu_workspace_bytes(int T, int I, int K, int dtype) {
+  if (T <= 0 || I <= 0 || K <= 0) return 0;
+  if (dtype == ODY_BF16 && T % 256 == 0 && I % 256 == 0 && K % BK == 0) return 0;
+  return (((size_t)T * I * (dtype == ODY_BF16 ? 2 : 4)) + 255) & ~(size_t)255;
+}
+
+extern "C" int ody_linear_dgrad_swiglu(const void* dy, const void* w_down, const void* gate_up, void* d_gate_up, int T,
+                                       int I, int K, int64_t ld_dy, int64_t ldw, int64_t ld_gu, int64_t ld_dgu, int dtype,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_lin("ody_linear_dgrad_swiglu", dy, w_down, d_gate_up, T, I, K, dtype);
+  if (rc) return rc;
+  ODY_REQUIRE(gate_up != nullptr, ODY_ERR_NULL, "ody_linear_dgrad_swiglu: gate_up is NULL");
+  ODY_REQUIRE(ld_dy >= K && ldw >= I && ld_gu >= 2 * (int64_t)I && ld_dgu >= 2 * (int64_t)I, ODY_ERR_BAD_SHAPE,
+              "ody_linear_dgrad_swiglu: leading dimension smaller than the row length");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && fused_shape_ok(T, I, K, ld_dy, ldw) && vec16(dy, ld_dy) && vec16(w_down, ldw) &&
+      vec16(gate_up, ld_gu) && vec16(d_gate_up, ld_dgu)) {
+    GemmEpi ep{static_cast<const bf16*>(gate_up), nullptr, ld_gu, 0, I};
+    return launch_fused<false, EPI_SWIGLU_BWD>("gemm_bf16_nn_swiglu_bwd", static_cast<const bf16*>(dy),
+                                               static_cast<const bf16*>(w_down), static_cast<bf16*>(d_gate_up), T, I, K,
+                                               ld_dy, ldw, ld_dgu, ep, st);
+  }
+  const size_t need = (size_t)T * I * (dtype == ODY_BF16 ? 2 : 4);
+  ODY_REQUIRE(workspace != nullptr && workspace_bytes >= need && ody_aligned16(workspace), ODY_ERR_WORKSPACE,
+              "ody_linear_dgrad_swiglu: this shape runs as two kernels and needs a 16-byte aligned workspace of %zu bytes "
+              "for dh (got %zu)", need, workspace ? workspace_bytes : (size_t)0);
+  rc = ody_gemm(ODY_GEMM_NN, dy, w_down, workspace, nullptr, T, I, K, ld_dy, ldw, I, 0, dtype, nullptr, 0, stream);
+  if (rc) return rc;
+  return ody_swiglu_bwd(gate_up, workspace, d_gate_up, T, I, ld_gu, I, ld_dgu, dtype, stream);
 }

@@ -169,10 +169,25 @@ class LlamaFlashAttention2TPSP(nn.Module):
             attn_output = ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
 
         attn_output = attn_output.reshape(bsz, q_len, nh * D)
-        attn_output = self.o_proj(attn_output)
+        residual = kwargs.get("residual")
+        if residual is not None and self._can_fuse_residual(residual, attn_output):
+            # the caller's skip connection rides in the output projection's epilogue
+            attn_output = ops.LinearResidualFunc.apply(attn_output, self.o_proj.weight, residual)
+        else:
+            attn_output = self.o_proj(attn_output)
+            if residual is not None:
+                attn_output = residual + attn_output
         if self.return_arity == 2:
             return attn_output, None
         return attn_output, None, past_key_value
+
+    def _can_fuse_residual(self, residual, attn_output) -> bool:
+        """The epilogue add stands for reduce_scatter(x W^T) + residual, which is only the same thing when the
+        reduce-scatter is the identity (one rank), there is no bias (it is added after the scatter) and
+        autocast does not ask for a cast."""
+        return (get_model_parallel_world_size() == 1 and self.o_proj.bias is None and self.o_proj.input_is_parallel
+                and residual.dtype == attn_output.dtype == self.o_proj.weight.dtype
+                and not torch.is_autocast_enabled("cuda"))
 
     def _update_cache(self, cache, k, v, q_len, cache_position):
         """Hands the rotated keys and the values of a prefill to the caller's cache, as
@@ -201,9 +216,17 @@ class LlamaMLPZeRO(nn.Module):
             raise NotImplementedError(f"hidden_act={act!r}: only the SiLU gate of Llama is implemented")
         self.act_fn = torch.nn.functional.silu  # kept as an attribute for introspection; the fused kernel applies it
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """`residual` (an extension: the reference's module takes x only) makes the result
+        residual + mlp(x) with every elementwise step fused into the products' epilogues."""
         if getattr(self.config, "pretraining_tp", 1) > 1:
             raise NotImplementedError("pretraining_tp > 1 is not supported yet.")
+        if residual is not None:
+            w1, w2 = self.gate_up_proj.weight, self.down_proj.weight
+            if (get_model_parallel_world_size() == 1 and self.gate_up_proj.bias is None and self.down_proj.bias is None
+                    and x.dtype == residual.dtype == w1.dtype == w2.dtype and not torch.is_autocast_enabled("cuda")):
+                return ops.SwiGLUMLPResidualFunc.apply(x, w1, w2, residual)
+            return residual + self.down_proj(ops.swiglu(self.gate_up_proj(x)))
         return self.down_proj(ops.swiglu(self.gate_up_proj(x)))
 
 
@@ -221,10 +244,17 @@ class LlamaRMSNorm(nn.Module):
 
 
 class OdysseusDecoderLayer(nn.Module):
-    """h = x + attn(rms(x)); y = h + mlp(rms(h)) (the wiring at decoder/ring.py:65-86)."""
+    """h = x + attn(rms(x)); y = h + mlp(rms(h)) (the wiring at decoder/ring.py:65-86).
 
-    def __init__(self, config, layer_idx: int = 0):
+    fused=True (default) runs the same arithmetic with the memory-bound steps folded into their
+    neighbours: both residual adds in the epilogues of the output / down projections, SwiGLU and its
+    backward in the epilogues of the gate_up product and of the down projection's input gradient, and
+    the sum of the two gradients at each fork of the residual stream inside the RMSNorm backward.
+    fused=False keeps one kernel per step, as the reference's layer does."""
+
+    def __init__(self, config, layer_idx: int = 0, fused: bool = True):
         super().__init__()
+        self.fused = fused
         self.hidden_size = config.hidden_size
         eps = getattr(config, "rms_norm_eps", 1e-6)
         self.self_attn = LlamaFlashAttention2TPSP(config, layer_idx)
@@ -233,6 +263,12 @@ class OdysseusDecoderLayer(nn.Module):
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
 
     def forward(self, hidden_states, attention_mask=None, position_ids=None, **kwargs):
+        if self.fused:
+            n1, skip = ops.rmsnorm_fork(hidden_states, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
+            h = self.self_attn(n1, attention_mask=attention_mask, position_ids=position_ids, residual=skip)[0]
+            n2, skip = ops.rmsnorm_fork(h, self.post_attention_layernorm.weight,
+                                        self.post_attention_layernorm.variance_epsilon)
+            return self.mlp(n2, residual=skip)
         residual = hidden_states
         hidden_states = self.self_attn(self.input_layernorm(hidden_states), attention_mask=attention_mask,
                                        position_ids=position_ids)[0]

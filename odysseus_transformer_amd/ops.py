@@ -190,6 +190,60 @@ def gemm(op: int, a, b, bias=None, out=None, accumulate: bool = False):
     return out
 
 
+def _lin_args(x, w, name):
+    if x.dim() != 2 or w.dim() != 2 or x.stride(1) != 1 or w.stride(1) != 1:
+        raise ValueError(f"{name}: 2-D row-major operands expected, got {tuple(x.shape)} {x.stride()} and "
+                         f"{tuple(w.shape)} {w.stride()}")
+    if x.dtype != w.dtype or x.device != w.device:
+        raise TypeError(f"{name}: operands differ in dtype or device ({x.dtype} {x.device} vs {w.dtype} {w.device})")
+
+
+def linear_residual(x, weight, residual):
+    """x (M, K) W (N, K)^T + residual (M, N), the add in the product's epilogue."""
+    _need_gpu(x, weight, residual)
+    _lin_args(x, weight, "linear_residual")
+    (M, K), N = x.shape, weight.shape[0]
+    if weight.shape[1] != K or tuple(residual.shape) != (M, N) or residual.dtype != x.dtype or residual.stride(1) != 1:
+        raise ValueError(f"linear_residual: x {tuple(x.shape)}, weight {tuple(weight.shape)}, residual "
+                         f"{tuple(residual.shape)} {residual.dtype} do not fit")
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    _lib.call("ody_linear_residual", x.data_ptr(), weight.data_ptr(), residual.data_ptr(), y.data_ptr(), M, N, K,
+              _rowmajor2d(x, "x"), _rowmajor2d(weight, "weight"), _rowmajor2d(residual, "residual"), y.stride(0),
+              _dt(x), _stream())
+    return y
+
+
+def linear_swiglu(x, w_gate_up):
+    """gate_up = x (T, K) Wgu (2 I, K)^T and h = silu(gate) * up in one kernel -> (gate_up, h)."""
+    _need_gpu(x, w_gate_up)
+    _lin_args(x, w_gate_up, "linear_swiglu")
+    (T, K), I2 = x.shape, w_gate_up.shape[0]
+    if w_gate_up.shape[1] != K or I2 % 2:
+        raise ValueError(f"linear_swiglu: x {tuple(x.shape)} and the packed weight {tuple(w_gate_up.shape)} do not fit")
+    gate_up = torch.empty((T, I2), dtype=x.dtype, device=x.device)
+    h = torch.empty((T, I2 // 2), dtype=x.dtype, device=x.device)
+    _lib.call("ody_linear_swiglu", x.data_ptr(), w_gate_up.data_ptr(), gate_up.data_ptr(), h.data_ptr(), T, I2 // 2, K,
+              _rowmajor2d(x, "x"), _rowmajor2d(w_gate_up, "w_gate_up"), gate_up.stride(0), h.stride(0), _dt(x), _stream())
+    return gate_up, h
+
+
+def linear_dgrad_swiglu(dy, w_down, gate_up):
+    """d_gate_up from dy (T, K) and the down weight (K, I): dh = dy Wd never leaves the kernel."""
+    _need_gpu(dy, w_down, gate_up)
+    _lin_args(dy, w_down, "linear_dgrad_swiglu")
+    (T, K), I = dy.shape, w_down.shape[1]
+    if w_down.shape[0] != K or tuple(gate_up.shape) != (T, 2 * I) or gate_up.dtype != dy.dtype or gate_up.stride(1) != 1:
+        raise ValueError(f"linear_dgrad_swiglu: dy {tuple(dy.shape)}, w_down {tuple(w_down.shape)}, gate_up "
+                         f"{tuple(gate_up.shape)} {gate_up.dtype} do not fit")
+    dgu = torch.empty((T, 2 * I), dtype=dy.dtype, device=dy.device)
+    ws_bytes = _lib.load().ody_linear_dgrad_swiglu_workspace_bytes(T, I, K, _dt(dy))
+    ws = scratch(ws_bytes, "dgrad_swiglu_workspace", dy.device) if ws_bytes else None
+    _lib.call("ody_linear_dgrad_swiglu", dy.data_ptr(), w_down.data_ptr(), gate_up.data_ptr(), dgu.data_ptr(), T, I, K,
+              _rowmajor2d(dy, "dy"), _rowmajor2d(w_down, "w_down"), _rowmajor2d(gate_up, "gate_up"), dgu.stride(0),
+              _dt(dy), ws.data_ptr() if ws is not None else 0, ws_bytes, _stream())
+    return dgu
+
+
 # --------------------------------------------------------------------------- elementwise
 def swiglu_fwd(gate_up):
     _need_gpu(gate_up)
@@ -264,18 +318,26 @@ def rmsnorm_fwd(x, weight, eps: float = 1e-6):
     return y.view(x.shape), rstd
 
 
-def rmsnorm_bwd(x, weight, rstd, dy):
-    _need_gpu(x, weight, rstd, dy)
+def rmsnorm_bwd(x, weight, rstd, dy, dx_add=None):
+    """dx, dw of rmsnorm; `dx_add` (same shape as x) is added to dx inside the kernel: the
+    gradient that reaches the norm's input over the residual connection."""
+    _need_gpu(x, weight, rstd, dy, dx_add)
     check_rmsnorm_args(x, weight, rstd, dy)
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
     dy2 = dy.reshape(-1, dy.shape[-1]).contiguous()
+    add_ptr = 0
+    if dx_add is not None:
+        if dx_add.dtype != x.dtype or dx_add.shape != x.shape or dx_add.device != x.device:
+            raise ValueError(f"rmsnorm: dx_add must match x ({tuple(x.shape)}, {x.dtype}, {x.device})")
+        dx_add = dx_add.reshape(-1, x.shape[-1]).contiguous()
+        add_ptr = dx_add.data_ptr()
     T, d = x2.shape
     dx = torch.empty_like(x2)
     dw = torch.empty_like(weight)
     nparts = _lib.load().ody_rmsnorm_bwd_partials(T)
     partial = scratch(nparts * d * 4, "rmsnorm_dw_partials", x.device)
-    _lib.call("ody_rmsnorm_bwd", x2.data_ptr(), weight.data_ptr(), rstd.data_ptr(), dy2.data_ptr(), dx.data_ptr(),
-              partial.data_ptr(), dw.data_ptr(), T, d, _dt(x2), _stream())
+    _lib.call("ody_rmsnorm_bwd", x2.data_ptr(), weight.data_ptr(), rstd.data_ptr(), dy2.data_ptr(), add_ptr,
+              dx.data_ptr(), partial.data_ptr(), dw.data_ptr(), T, d, _dt(x2), _stream())
     return dx.view(x.shape), dw
 
 
@@ -432,8 +494,82 @@ class RoPEFunc(torch.autograd.Function):
         return dx, None, None, None
 
 
+class RMSNormForkFunc(torch.autograd.Function):
+    """(norm(x), x): the point where the residual stream forks into a normalised branch and the skip
+    connection.  Autograd would add the two gradients that come back with a kernel of its own; here the
+    skip gradient goes into the norm's backward kernel as `dx_add`."""
+
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        y, rstd = rmsnorm_fwd(x, weight, eps)
+        ctx.save_for_backward(x, weight, rstd)
+        ctx.set_materialize_grads(False)
+        return y, x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, dy, dskip):
+        x, weight, rstd = ctx.saved_tensors
+        if dy is None:
+            return dskip, None, None
+        dx, dw = rmsnorm_bwd(x, weight, rstd, dy, dx_add=dskip)
+        return dx, dw, None
+
+
+class LinearResidualFunc(torch.autograd.Function):
+    """residual + x W^T with the add in the product's epilogue; backward: dX = dY W, dW = dY^T X and
+    the residual's gradient is dY itself."""
+
+    @staticmethod
+    def forward(ctx, x, weight, residual):
+        ctx.save_for_backward(x, weight)
+        y = linear_residual(x.reshape(-1, x.shape[-1]), weight, residual.reshape(-1, residual.shape[-1]))
+        return y.view(residual.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        dy2 = dy2 if dy2.stride(1) == 1 else dy2.contiguous()
+        dx = gemm(GEMM_NN, dy2, weight).view(x.shape)
+        x2 = x.reshape(-1, x.shape[-1])
+        dw = gemm(GEMM_TN, dy2, x2 if x2.stride(1) == 1 else x2.contiguous())
+        return dx, dw, dy
+
+
+class SwiGLUMLPResidualFunc(torch.autograd.Function):
+    """residual + down(silu(gate) * up) with gate_up = x Wgu^T, every elementwise step inside a product's
+    epilogue: SwiGLU in the gate_up product, the residual add in the down product, the SwiGLU backward
+    in the down product's input gradient (decoder/odysseus.py:293-295 and the add at decoder/ring.py:86)."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate_up, w_down, residual):
+        x2 = x.reshape(-1, x.shape[-1])
+        x2 = x2 if x2.stride(1) == 1 else x2.contiguous()
+        gate_up, h = linear_swiglu(x2, w_gate_up)
+        y = linear_residual(h, w_down, residual.reshape(-1, residual.shape[-1]))
+        ctx.save_for_backward(x2, w_gate_up, w_down, gate_up, h)
+        ctx.x_shape = x.shape
+        return y.view(residual.shape)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x2, w_gate_up, w_down, gate_up, h = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.shape[-1])
+        dy2 = dy2 if dy2.stride(1) == 1 else dy2.contiguous()
+        dw_down = gemm(GEMM_TN, dy2, h)
+        dgu = linear_dgrad_swiglu(dy2, w_down, gate_up)
+        dx = gemm(GEMM_NN, dgu, w_gate_up).view(ctx.x_shape)
+        dw_gate_up = gemm(GEMM_TN, dgu, x2)
+        return dx, dw_gate_up, dw_down, dy
+
+
 def rmsnorm(x, weight, eps: float = 1e-6):
     return RMSNormFunc.apply(x, weight, eps)
+
+
+def rmsnorm_fork(x, weight, eps: float = 1e-6):
+    """-> (rmsnorm(x), x) with the two returning gradients summed inside the norm's backward kernel."""
+    return RMSNormForkFunc.apply(x, weight, eps)
 
 
 def swiglu(gate_up):

@@ -29,6 +29,17 @@ def test_rmsnorm(T, d, dtype, dev):
         dx, dw = ops.rmsnorm_bwd(x.to(dev), w.to(dev), rstd, dy.to(dev))
         assert rel_err(dx, dx_ref) <= _tol(dtype)
         assert rel_err(dw, dw_ref) <= _tol(dtype)
+        # with the gradient of the residual path added inside the kernel
+        skip = randn((1, T, d), 4, dtype=dtype)
+        dx2, dw2 = ops.rmsnorm_bwd(x.to(dev), w.to(dev), rstd, dy.to(dev), dx_add=skip.to(dev))
+        assert rel_err(dx2, dx_ref.float() + skip.float()) <= _tol(dtype)
+        assert torch.equal(dw2, dw)
+    else:
+        # rows longer than the backward kernel holds in registers are refused, not mangled
+        from odysseus_transformer_amd._lib import OdysseusHipError
+        with pytest.raises(OdysseusHipError) as e:
+            ops.rmsnorm_bwd(x.to(dev), w.to(dev), rstd, dy.to(dev))
+        assert e.value.code == -2
 
 
 @DTYPES
