@@ -123,11 +123,18 @@ int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out,
  * gradients sum to the gradient of the unsplit attention.
  * dq/dk/dv have the shapes of q/k/v with their own strides.  dK and dV of a kv
  * head are summed over its query-head group inside the kernel (deterministic,
- * no atomics).  If accumulate_dq != 0 the kernel adds into dq (fp32 dq_accum
- * layout not needed: the add happens in fp32 before rounding once).
+ * no atomics).  `flags` is a sum of
+ *   ODY_BWD_ACCUMULATE_DQ     the kernel adds into dq (in fp32, rounded once per call when dq is bf16);
+ *   ODY_BWD_DQ_F32            dq is an fp32 buffer (strides in fp32 elements) although q is bf16: with
+ *                             ACCUMULATE this is the ring step's running dq, exact over any number of key
+ *                             blocks and rounded once by the caller at the end (ody_cast_from_f32);
+ *   ODY_BWD_REUSE_QUERY_SIDE  q, out, lse, dout and the workspace are those of the previous call: delta and
+ *                             the other query-side scratch in the workspace are taken as they are (the ring
+ *                             step calls once per key block with the same queries).
  * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
- * the bf16 head_dim-128 kernels a transposed copy of K).
+ * the bf16 head_dim-128 kernels transposed copies of K, Q and dO).
  */
+enum ody_attn_bwd_flags { ODY_BWD_ACCUMULATE_DQ = 1, ODY_BWD_DQ_F32 = 2, ODY_BWD_REUSE_QUERY_SIDE = 4 };
 size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
                  const void* dout, void* dq, void* dk, void* dv,
@@ -140,7 +147,7 @@ int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, c
                  int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
                  int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
                  int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
-                 float scale, int causal, int accumulate_dq, int dtype,
+                 float scale, int causal, int flags, int dtype,
                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* Online-softmax merge of one key block's partial result into the running one
@@ -154,6 +161,11 @@ int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, c
 int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk, const float* lse_blk,
                   int B, int L, int H, int D, int64_t sb_b, int64_t sb_l, int64_t sb_h,
                   int dtype, void* stream);
+
+/* Rounds an fp32 array to `dtype` (n elements, both 16-byte aligned, n a multiple of 8): the last step of a
+ * result that was accumulated in fp32 over the key blocks of a ring step (running out, running dq).
+ */
+int ody_cast_from_f32(const float* src, void* dst, int64_t n, int dtype, void* stream);
 
 /* ---- dense linears ------------------------------------------------------
  * C (M, N) = op(A) * op(B), row-major, leading dimensions in elements.

@@ -145,15 +145,19 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
                             int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
                             int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
                             int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
-                            float scale, int causal, int accumulate_dq, int dtype,
+                            float scale, int causal, int flags, int dtype,
                             void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common("ody_attn_bwd", B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
+  ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE)) == 0, ODY_ERR_UNSUPPORTED,
+              "ody_attn_bwd: unknown flag bits in %d", flags);
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
   p.dout = dout; p.dq = dq; p.dk = dk; p.dv = dv;
   p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
-  p.causal = causal ? 1 : 0; p.off = Lk - Lq; p.accumulate_dq = accumulate_dq ? 1 : 0;
+  p.causal = causal ? 1 : 0; p.off = Lk - Lq; p.accumulate_dq = (flags & ODY_BWD_ACCUMULATE_DQ) ? 1 : 0;
+  p.dq_f32 = (flags & ODY_BWD_DQ_F32) || dtype == ODY_F32 ? 1 : 0;
+  p.reuse_query_side = (flags & ODY_BWD_REUSE_QUERY_SIDE) ? 1 : 0;
   p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
   p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
   p.sdo = {sdo_b, sdo_l, sdo_h}; p.sdq = {sdq_b, sdq_l, sdq_h}; p.sdk = {sdk_b, sdk_l, sdk_h};
@@ -165,7 +169,7 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
   if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "out", out, p.so, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "dq", dq, p.sdq, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dq", dq, p.sdq, p.dq_f32 ? ODY_F32 : dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dk", dk, p.sdk, dtype, vec))) return rc;
   if ((rc = check_tensor(who, "dv", dv, p.sdv, dtype, vec))) return rc;
   ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_bwd: lse is NULL");
@@ -178,7 +182,7 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
               "ody_attn_bwd: workspace must be 256-byte aligned");
   p.delta = static_cast<float*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if ((rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
+  if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
   if (dtype == ODY_BF16 && D == 128)
     return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
   if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);

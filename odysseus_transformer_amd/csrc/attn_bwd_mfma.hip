@@ -320,7 +320,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
     __syncthreads();
   }
 
-  if (qi < p.Lq) {
+  if (qi < p.Lq && p.dq_f32) {
+    float* dqp = static_cast<float*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        f32x4* dst = reinterpret_cast<f32x4*>(dqp + 32 * dt + 8 * a + 4 * g);
+        f32x4 w = {0.f, 0.f, 0.f, 0.f};
+        if (p.accumulate_dq) w = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] += dq[dt][4 * a + e] * p.scale;
+        *dst = w;
+      }
+  } else if (qi < p.Lq) {
     bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)

@@ -204,7 +204,21 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 #pragma unroll
   for (int qt = 0; qt < QT; qt++) {
     const int qi = wq0 + 32 * qt + i;
-    if (qi < p.Lq) {
+    if (qi < p.Lq && p.dq_f32) {
+      // fp32 destination (the ring step's running dq): exact accumulation over the key blocks, no rounding here
+      float* dqp = static_cast<float*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          f32x4* dst = reinterpret_cast<f32x4*>(dqp + 32 * dt + 8 * a + 4 * g);
+          f32x4 w = {0.f, 0.f, 0.f, 0.f};
+          if (p.accumulate_dq) w = *dst;
+#pragma unroll
+          for (int e = 0; e < 4; e++) w[e] += dq[qt][dt][4 * a + e] * p.scale;
+          *dst = w;
+        }
+    } else if (qi < p.Lq) {
       bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
@@ -516,12 +530,14 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   bf16* stats = reinterpret_cast<bf16*>(reinterpret_cast<unsigned char*>(doimg) +
                                         align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
   int rc;
-  ODY_LAUNCH("attn_bwd_stats", st, attn_bwd_stats_kernel, dim3((p.Lq + KV_BQ - 1) / KV_BQ, p.Hq, p.B), dim3(128), 0, p,
-             stats);
-  if ((rc = ody_check_launch("attn_bwd_stats"))) return rc;
+  if (!p.reuse_query_side) {   // everything that depends on q, dout, out and lse only
+    ODY_LAUNCH("attn_bwd_stats", st, attn_bwd_stats_kernel, dim3((p.Lq + KV_BQ - 1) / KV_BQ, p.Hq, p.B), dim3(128), 0, p,
+               stats);
+    if ((rc = ody_check_launch("attn_bwd_stats"))) return rc;
+    if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
+    if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
+  }
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
-  if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
-  if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
   const int key_blocks = (p.Lk + KV_BN - 1) / KV_BN;
   if (p.group == 1) {
     ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<false>, dim3(key_blocks * p.Hkv * p.B),

@@ -21,6 +21,8 @@ struct AttnParams {
   int causal;         // 0/1
   int off;            // Lk - Lq: key j visible to query i iff j <= i + off
   int accumulate_dq;  // bwd: dq += result
+  int dq_f32;         // bwd: dq is an fp32 buffer (strides in fp32 elements) whatever the storage type of q
+  int reuse_query_side;  // bwd: delta, start values and the Q / dO images in the workspace are those of the previous call
   float scale;        // softmax scale
   float scale_log2e;  // scale * log2(e)
   AttnStrides sq, sk, sv, so, sdo, sdq, sdk, sdv;

@@ -401,6 +401,36 @@ extern "C" int ody_rope(void* x, const int64_t* position_ids, const float* inv_f
   return ody_check_launch("rope");
 }
 
+namespace {
+__global__ __launch_bounds__(256) void cast_from_f32_kernel(const float* __restrict__ src, bf16* __restrict__ dst,
+                                                            int64_t n8) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n8) return;
+  const f32x4 a = *reinterpret_cast<const f32x4*>(src + idx * 8), b = *reinterpret_cast<const f32x4*>(src + idx * 8 + 4);
+  bf16x8 w;
+#pragma unroll
+  for (int e = 0; e < 4; e++) w[e] = (bf16)a[e], w[4 + e] = (bf16)b[e];
+  *reinterpret_cast<bf16x8*>(dst + idx * 8) = w;
+}
+}  // namespace
+
+extern "C" int ody_cast_from_f32(const float* src, void* dst, int64_t n, int dtype, void* stream) {
+  ODY_REQUIRE(src && dst, ODY_ERR_NULL, "ody_cast_from_f32: NULL pointer");
+  ODY_REQUIRE(n > 0 && n % 8 == 0, ODY_ERR_BAD_SHAPE, "ody_cast_from_f32: n=%lld must be a positive multiple of 8", (long long)n);
+  ODY_REQUIRE(ody_aligned16(src) && ody_aligned16(dst), ODY_ERR_MISALIGNED, "ody_cast_from_f32: 16-byte alignment required");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_F32) {
+    if (static_cast<const void*>(src) == dst) return ODY_OK;
+    hipError_t e = hipMemcpyAsync(dst, src, (size_t)n * sizeof(float), hipMemcpyDeviceToDevice, st);
+    ODY_REQUIRE(e == hipSuccess, ODY_ERR_LAUNCH, "ody_cast_from_f32: copy failed: %s", hipGetErrorString(e));
+    return ODY_OK;
+  }
+  ODY_REQUIRE(dtype == ODY_BF16, ODY_ERR_UNSUPPORTED, "ody_cast_from_f32: dtype %d unknown", dtype);
+  ODY_LAUNCH("cast_from_f32", st, cast_from_f32_kernel, dim3(blocks_for(n / 8)), dim3(256), 0, src, static_cast<bf16*>(dst),
+             n / 8);
+  return ody_check_launch("cast_from_f32");
+}
+
 extern "C" int ody_swiglu_fwd(const void* gate_up, void* h, int T, int I, int64_t ld_gu, int64_t ld_h, int dtype,
                               void* stream) {
   ODY_REQUIRE(gate_up && h, ODY_ERR_NULL, "ody_swiglu_fwd: NULL pointer");

@@ -110,8 +110,13 @@ def attn_fwd_noalloc(q, k, v, out, lse, causal: bool = True, scale: Optional[flo
 
 
 def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
-             dq=None, dk=None, dv=None, accumulate_dq: bool = False):
-    """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step."""
+             dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False):
+    """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.
+
+    dq may be a float32 tensor although q is bfloat16: with accumulate_dq that is the running dq of a
+    ring step, summed exactly over the key blocks.  reuse_query_side=True (needs the `workspace` of
+    the previous call, with the same q / out / lse / dout) skips the scratch that depends on the
+    queries only."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
@@ -121,22 +126,55 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
         dq = torch.empty_like(q)
     dk = torch.empty_like(k) if dk is None else dk
     dv = torch.empty_like(v) if dv is None else dv
-    _same(q, "q", out=out, dout=dout, dq=dq)
+    dq_f32 = dq.dtype == torch.float32 and q.dtype != torch.float32
+    _same(q, "q", out=out, dout=dout)
+    if dq.shape != q.shape or dq.device != q.device or (dq.dtype != q.dtype and not dq_f32):
+        raise ValueError(f"dq must have q's shape and device and q's dtype or float32; got {tuple(dq.shape)} {dq.dtype}")
     _same(k, "k", v=v, dk=dk, dv=dv)
     if k.dtype != q.dtype or k.shape[0] != B or k.shape[3] != D or tuple(lse.shape) != (B, Hq, Lq):
         raise ValueError(f"k {tuple(k.shape)} {k.dtype} / lse {tuple(lse.shape)} do not match q {tuple(q.shape)} {q.dtype}")
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     lib = _lib.load()
     ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
-    ws = scratch(ws_bytes, "attn_bwd_workspace", q.device)
+    if workspace is None:
+        if reuse_query_side:
+            raise ValueError("reuse_query_side needs the workspace of the previous call")
+        ws = scratch(ws_bytes, "attn_bwd_workspace", q.device)
+    else:
+        ws = workspace
+        if ws.dtype != torch.uint8 or ws.numel() < ws_bytes or ws.device != q.device or not ws.is_contiguous():
+            raise ValueError(f"workspace must be a contiguous uint8 tensor of at least {ws_bytes} bytes on {q.device}")
+    flags = (_lib.BWD_ACCUMULATE_DQ if accumulate_dq else 0) | (_lib.BWD_DQ_F32 if dq_f32 else 0) | \
+            (_lib.BWD_REUSE_QUERY_SIDE if reuse_query_side else 0)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
     _lib.call("ody_attn_bwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
               dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
               B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
               *_blhd(dout, "dout"), *_blhd(dq, "dq"), *_blhd(dk, "dk"), *_blhd(dv, "dv"),
-              scale, int(causal), int(accumulate_dq), _dt(q), ws.data_ptr(), ws_bytes, _stream())
+              scale, int(causal), flags, _dt(q), ws.data_ptr(), ws_bytes, _stream())
     return dq, dk, dv
+
+
+def attn_bwd_workspace(q, k) -> torch.Tensor:
+    """A workspace for attn_bwd on these shapes, for callers that make several calls with the same queries."""
+    B, Lq, Hq, D = q.shape
+    n = _lib.load().ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q))
+    return torch.empty(n, dtype=torch.uint8, device=q.device)
+
+
+def cast_from_f32(src, dtype) -> torch.Tensor:
+    """Rounds a contiguous float32 tensor to `dtype` (the end of an fp32 accumulation over ring blocks)."""
+    _need_gpu(src)
+    if src.dtype != torch.float32 or not src.is_contiguous():
+        raise ValueError("cast_from_f32 takes a contiguous float32 tensor")
+    if dtype == torch.float32:
+        return src
+    dst = torch.empty(src.shape, dtype=dtype, device=src.device)
+    if src.numel() % 8:
+        return dst.copy_(src)
+    _lib.call("ody_cast_from_f32", src.data_ptr(), dst.data_ptr(), src.numel(), _dt(dst), _stream())
+    return dst
 
 
 def lse_merge_(out_acc, lse_acc, out_blk, lse_blk) -> None:
@@ -409,7 +447,7 @@ class RingBlocksAttnFunc(torch.autograd.Function):
         for b in range(nb):
             ob, lb = attn_fwd(q, ks[b], vs[b], causal=(b == causal_block), scale=softmax_scale)
             lse_merge_(acc, lse, ob, lb)
-        out = acc.to(q.dtype)
+        out = cast_from_f32(acc, q.dtype)
         ctx.save_for_backward(q, out, lse, *kv)
         ctx.causal_block, ctx.softmax_scale = causal_block, softmax_scale
         ctx.mark_non_differentiable(lse)
@@ -422,14 +460,19 @@ class RingBlocksAttnFunc(torch.autograd.Function):
         ks, vs = kv[:nb], kv[nb:]
         if dout.stride(3) != 1:
             dout = dout.contiguous()
-        dq = torch.empty_like(q)
+        # the running dq stays in fp32 over the blocks and is rounded once; delta, the start values and the
+        # Q / dO images depend on the queries only and are built by the first block's call
+        dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+        same_kv_shape = all(k.shape == ks[0].shape for k in ks)
+        ws = attn_bwd_workspace(q, max(ks, key=lambda t: t.shape[1])) if nb else None
         dks, dvs = [], []
         for b in range(nb):
             _, dk, dv = attn_bwd(q, ks[b], vs[b], out, lse, dout, causal=(b == ctx.causal_block),
-                                 scale=ctx.softmax_scale, dq=dq, accumulate_dq=(b > 0))
+                                 scale=ctx.softmax_scale, dq=dq, accumulate_dq=(b > 0), workspace=ws,
+                                 reuse_query_side=(b > 0 and same_kv_shape))
             dks.append(dk)
             dvs.append(dv)
-        return (dq, None, None, *dks, *dvs)
+        return (cast_from_f32(dq, q.dtype), None, None, *dks, *dvs)
 
 
 def ring_blocks_attn(q, k_blocks, v_blocks, causal_block: Optional[int] = 0, softmax_scale: Optional[float] = None):

@@ -155,6 +155,41 @@ def test_ring_step_equals_unsplit_attention(dev):
     assert_parity(torch.cat(dvs[1:] + dvs[:1], 1), dv_ref, TOL_BF16, "dv")
 
 
+def test_ring_backward_fp32_dq_and_reused_query_side(dev):
+    """Over many key blocks the bf16 running dq is rounded after every block; the fp32 one is exact and is
+    rounded once.  Reusing the query-side scratch of the first block's call changes nothing."""
+    from odysseus_transformer_amd import ops
+    B, Lq, H, D, NB = 1, 320, 2, 128, 6
+    dt = torch.bfloat16
+    q, do = randn((B, Lq, H, D), 70, dtype=dt), randn((B, Lq, H, D), 71, dtype=dt)
+    ks = [randn((B, 192, H, D), 72 + b, dtype=dt) for b in range(NB)]
+    vs = [randn((B, 192, H, D), 82 + b, dtype=dt) for b in range(NB)]
+    o_ref, l_ref = oracle.ring_attention_fwd(q.float(), [k.float() for k in ks], [v.float() for v in vs], causal_block=None)
+    dq_ref, dk_ref, dv_ref = oracle.ring_attention_bwd(q.float(), [k.float() for k in ks], [v.float() for v in vs], o_ref,
+                                                       l_ref, do.float(), causal_block=None)
+    qg, dog = q.to(dev), do.to(dev)
+    kg, vg = [k.to(dev) for k in ks], [v.to(dev) for v in vs]
+    out, lse = o_ref.to(dt).to(dev), l_ref.to(dev)
+    runs = {}
+    for name, f32, reuse in (("bf16", False, False), ("fp32", True, False), ("fp32_reuse", True, True)):
+        dq = torch.empty(qg.shape, dtype=torch.float32 if f32 else dt, device=dev)
+        ws = ops.attn_bwd_workspace(qg, kg[0])
+        dks = []
+        for b in range(NB):
+            _, dk, _ = ops.attn_bwd(qg, kg[b], vg[b], out, lse, dog, causal=False, dq=dq, accumulate_dq=(b > 0),
+                                    workspace=ws, reuse_query_side=(reuse and b > 0))
+            dks.append(dk)
+        runs[name] = (dq.float().cpu(), dks)
+    assert torch.equal(runs["fp32"][0], runs["fp32_reuse"][0])
+    assert all(torch.equal(a, b) for a, b in zip(runs["fp32"][1], runs["fp32_reuse"][1]))
+    e_bf16, e_f32 = rel_err(runs["bf16"][0], dq_ref), rel_err(runs["fp32"][0], dq_ref)
+    assert e_f32 <= TOL_BF16 / 4 and e_f32 < e_bf16, (e_f32, e_bf16)
+    for b in range(NB):
+        assert_parity(runs["fp32"][1][b], dk_ref[b], TOL_BF16, f"dk block {b}")
+    with pytest.raises(ValueError):
+        ops.attn_bwd(qg, kg[0], vg[0], out, lse, dog, causal=False, reuse_query_side=True)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
 def test_ring_blocks_autograd_function(dtype, dev):
     """ops.ring_blocks_attn (forward merge + backward over blocks under autograd) vs. the oracle's ring loop."""

@@ -95,13 +95,18 @@ def test_cfg5_ring_of_eight_blocks_sampled(dev):
     for b in range(NB):
         ob, lb = ops.attn_fwd(qg, kg[b], vg[b], causal=(b == 0))
         ops.lse_merge_(out, lse, ob, lb)
-    out_bf = out.to(dt)
-    dq = torch.zeros_like(qg)
+    out_bf = ops.cast_from_f32(out, dt)
+    assert torch.equal(out_bf, out.to(dt))
+    # the running dq in fp32 over the 8 blocks; the query-side scratch (delta, Q / dO images) built once
+    dq32 = torch.empty(qg.shape, dtype=torch.float32, device=dev)
+    ws = ops.attn_bwd_workspace(qg, kg[0])
     dks, dvs = [], []
     for b in range(NB):
-        _, dk, dv = ops.attn_bwd(qg, kg[b], vg[b], out_bf, lse, dog, causal=(b == 0), dq=dq, accumulate_dq=(b > 0))
+        _, dk, dv = ops.attn_bwd(qg, kg[b], vg[b], out_bf, lse, dog, causal=(b == 0), dq=dq32, accumulate_dq=(b > 0),
+                                 workspace=ws, reuse_query_side=(b > 0))
         dks.append(dk.cpu())
         dvs.append(dv.cpu())
+    dq = ops.cast_from_f32(dq32, dt)
     torch.cuda.synchronize()
     order = list(range(1, NB)) + [0]
     cat = lambda ts: torch.cat([ts[b] for b in order], 1)[0]
