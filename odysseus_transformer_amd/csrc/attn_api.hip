@@ -182,9 +182,9 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
               "ody_attn_bwd: workspace must be 256-byte aligned");
   p.delta = static_cast<float*>(workspace);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
-  if (dtype == ODY_BF16 && D == 128)
+  if (dtype == ODY_BF16 && D == 128)   // its query-side pre-pass computes delta as well
     return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
+  if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
   if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
   return ody_launch_attn_bwd_f32(p, D, st);
 }

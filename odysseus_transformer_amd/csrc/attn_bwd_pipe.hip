@@ -250,32 +250,11 @@ constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 *
 constexpr int KV_STAT_ELEMS = 128 * 8;                                   // start-value fragments of one tile
 constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q, dO tiles; Q^T, dO^T images; start values
 
-// Pre-pass: the start values of S and dP for every 64-query tile, as one more A-operand
-// fragment of the contraction (the matching B fragment is all ones): the fp32 value x is split
-// into three bf16 terms x = h + m + l, which the MFMA adds up exactly like any other product.
-// Layout per (batch, head, tile): [sub-tile mt][0: -lse/scale, 1: -delta][MFMA row i][8 bf16],
-// row i of sub-tile mt being query tile_row(i, mt).  Rows that must give P = 0 (beyond Lq, or a
-// query that saw no key) get -1e30.
-__global__ __launch_bounds__(128) void attn_bwd_stats_kernel(const AttnParams p, bf16* __restrict__ stats) {
-  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int mt = threadIdx.x >> 6, which = (threadIdx.x >> 5) & 1, i = threadIdx.x & 31;
-  const int qi = t * KV_BQ + tile_row(i, mt);
-  const int64_t ri = ((int64_t)b * p.Hq + h) * p.Lq + qi;
-  float x;
-  if (which == 0) {
-    const float l = (qi < p.Lq) ? p.lse[ri] : INFINITY;
-    x = (l == INFINITY || l == -INFINITY) ? -1e30f : -l / p.scale;
-  } else {
-    x = (qi < p.Lq) ? -p.delta[ri] : 0.f;
-  }
-  const bf16 hi = (bf16)x;
-  const bf16 mid = (bf16)(x - (float)hi);
-  const bf16 lo = (bf16)(x - (float)hi - (float)mid);
-  const bf16 z = (bf16)0.f;
-  *reinterpret_cast<bf16x8*>(stats + ((((int64_t)b * p.Hq + h) * gridDim.x + t) * 128 + threadIdx.x) * 8) =
-      bf16x8{hi, mid, lo, z, z, z, z, z};
-}
-
+// The start values of S and dP for every 64-query tile enter as one more A-operand fragment of the contraction
+// (the matching B fragment is all ones): the fp32 value x is split into three bf16 terms x = h + m + l, which
+// the MFMA adds up exactly like any other product.  The query-side pre-pass (attn_bwd_prepass_kernel) writes
+// them: per (batch, head, tile) [sub-tile mt][0: -lse/scale, 1: -delta][MFMA row i][8 bf16], row i of sub-tile
+// mt being query tile_row(i, mt).  Rows that must give P = 0 (beyond Lq, or a query that saw no key) hold -1e30.
 //
 // SPLIT = false: a block owns 256 keys of one kv head and walks all query heads of its group.
 // SPLIT = true (grouped-query attention): a block owns 256 keys for ONE query head and writes
@@ -530,13 +509,8 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   bf16* stats = reinterpret_cast<bf16*>(reinterpret_cast<unsigned char*>(doimg) +
                                         align256(ody_attn_images_bytes(p.B, p.Lq, p.Hq)));
   int rc;
-  if (!p.reuse_query_side) {   // everything that depends on q, dout, out and lse only
-    ODY_LAUNCH("attn_bwd_stats", st, attn_bwd_stats_kernel, dim3((p.Lq + KV_BQ - 1) / KV_BQ, p.Hq, p.B), dim3(128), 0, p,
-               stats);
-    if ((rc = ody_check_launch("attn_bwd_stats"))) return rc;
-    if ((rc = ody_launch_attn_images(p.q, p.sq, p.B, p.Lq, p.Hq, qimg, nullptr, 0, st))) return rc;
-    if ((rc = ody_launch_attn_images(p.dout, p.sdo, p.B, p.Lq, p.Hq, doimg, nullptr, 0, st))) return rc;
-  }
+  // everything that depends on q, dout, out and lse only: delta, Q / dO images, start values
+  if (!p.reuse_query_side && (rc = ody_launch_attn_bwd_prepass(p, qimg, doimg, stats, st))) return rc;
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
   const int key_blocks = (p.Lk + KV_BN - 1) / KV_BN;
   if (p.group == 1) {

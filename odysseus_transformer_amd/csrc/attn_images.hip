@@ -42,7 +42,89 @@ __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict
   }
 }
 
+// The whole query side of the head_dim-128 backward in one pass over Q, dO and O (one block per 64-query tile of a
+// head): delta = sum_d dO * O, the transposed images of the Q tile and of the dO tile, and the tile's start-value
+// fragments (-lse / scale and -delta, each split into three bf16 terms; layout described where the dK/dV kernel reads
+// them).  Replaces four launches that each went over the same rows.
+__global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams p, bf16* __restrict__ qimg,
+                                                               bf16* __restrict__ doimg, bf16* __restrict__ stats) {
+  constexpr int PITCH = 128 + 8;
+  __shared__ __attribute__((aligned(16))) bf16 tq[64 * PITCH];
+  __shared__ __attribute__((aligned(16))) bf16 tdo[64 * PITCH];
+  __shared__ float sdelta[64];
+  const int tid = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z, ntiles = gridDim.x;
+  const bf16* qb = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h;
+  const bf16* dob = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
+  const bf16* ob = static_cast<const bf16*>(p.out) + b * p.so.b + h * p.so.h;
+  const bf16x8 zero = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int c = tid + 256 * j, row = c >> 4, col = (c & 15) * 8, gr = t * 64 + row;
+    bf16x8 qv = zero, dv = zero, ov = zero;
+    if (gr < p.Lq) {
+      qv = *reinterpret_cast<const bf16x8*>(qb + (int64_t)gr * p.sq.l + col);
+      dv = *reinterpret_cast<const bf16x8*>(dob + (int64_t)gr * p.sdo.l + col);
+      ov = *reinterpret_cast<const bf16x8*>(ob + (int64_t)gr * p.so.l + col);
+    }
+    *reinterpret_cast<bf16x8*>(tq + row * PITCH + col) = qv;
+    *reinterpret_cast<bf16x8*>(tdo + row * PITCH + col) = dv;
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc = fmaf((float)ov[e], (float)dv[e], acc);
+#pragma unroll
+    for (int sft = 8; sft > 0; sft >>= 1) acc += __shfl_xor(acc, sft, 64);   // the 16 lanes of one row
+    if ((tid & 15) == 0) {
+      sdelta[row] = acc;
+      if (gr < p.Lq) p.delta[((int64_t)b * p.Hq + h) * p.Lq + gr] = acc;
+    }
+  }
+  __syncthreads();
+  const int64_t tile_id = ((int64_t)b * p.Hq + h) * ntiles + t;
+#pragma unroll
+  for (int which = 0; which < 2; which++) {
+    const bf16* tile = which ? tdo : tq;
+    bf16* img = (which ? doimg : qimg) + tile_id * IMG_ELEMS;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int q = tid + 256 * j;                    // 16-byte chunk of the image
+      const int d = 16 * (q >> 7) + (q & 15), c = (q >> 4) & 7;
+      const int kt = c >> 2, ss = (c >> 1) & 1, g = c & 1;
+      bf16x8 v;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        const int row = 32 * (e >> 2) + 16 * g + 4 * (e & 3) + ss + 2 * kt;
+        v[e] = tile[row * PITCH + d];
+      }
+      *reinterpret_cast<bf16x8*>(img + q * 8) = v;
+    }
+  }
+  if (tid < 128) {
+    const int mt = tid >> 6, which = (tid >> 5) & 1, i = tid & 31;
+    const int row = tile_row(i, mt), qi = t * 64 + row;
+    float x;
+    if (which == 0) {
+      const float l = (qi < p.Lq) ? p.lse[((int64_t)b * p.Hq + h) * p.Lq + qi] : INFINITY;
+      x = (l == INFINITY || l == -INFINITY) ? -1e30f : -l / p.scale;
+    } else {
+      x = (qi < p.Lq) ? -sdelta[row] : 0.f;
+    }
+    const bf16 hi = (bf16)x;
+    const bf16 mid = (bf16)(x - (float)hi);
+    const bf16 lo = (bf16)(x - (float)hi - (float)mid);
+    const bf16 z = (bf16)0.f;
+    *reinterpret_cast<bf16x8*>(stats + (tile_id * 128 + tid) * 8) = bf16x8{hi, mid, lo, z, z, z, z, z};
+  }
+}
+
 }  // namespace
+
+int ody_launch_attn_bwd_prepass(const AttnParams& p, void* qimg, void* doimg, void* stats, hipStream_t st) {
+  dim3 grid((p.Lq + 63) / 64, p.Hq, p.B);
+  ODY_LAUNCH("attn_bwd_prepass", st, attn_bwd_prepass_kernel, grid, dim3(256), 0, p, static_cast<bf16*>(qimg),
+             static_cast<bf16*>(doimg), static_cast<bf16*>(stats));
+  return ody_check_launch("attn_bwd_prepass");
+}
 
 size_t ody_attn_images_bytes(int B, int L, int H) {
   return (size_t)B * H * ((L + 63) / 64) * tile128::IMG_BYTES;

@@ -197,18 +197,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
   }
   __syncthreads();
 
-  // Slab kt is in LDS buffer kt & 1 and the registers hold slab kt+1.  Per k-step a quarter of
-  // the registers goes to the other LDS buffer and is refilled at once with its part of slab kt+2.
+  // Slab kt is in LDS buffer kt & 1 and the registers hold slab kt+1.  During the first KSTEPS - 1 k-steps
+  // of a slab the staging registers go, one or two 16-byte chunks per group of WN MFMAs, to the other LDS
+  // buffer and are refilled at once with their part of slab kt+2.  The one barrier of the slab sits INSIDE
+  // the last k-step, behind its first group of MFMAs: by then every wavefront has written its part of slab
+  // kt+1 and has read its last fragments of slab kt, so the fragments of slab kt+1's first k-step can be
+  // fetched under the remaining MFMAs of slab kt instead of in front of an idle matrix pipe.
+  static_assert(CA == CB && KSTEPS > 1, "chunk schedule");
+  constexpr int MOVES = CA + CB, GROUPS = (KSTEPS - 1) * WM;
+  bf16x8 af[2][WM], bfr[2][WN];
+  if (nk > 0) {
+#pragma unroll
+    for (int a = 0; a < WM; a++) af[0][a] = TA::frag(As, 32 * (wm * WM + a), 0, g, i);
+#pragma unroll
+    for (int b = 0; b < WN; b++) bfr[0][b] = TB::frag(Bs, 32 * (wn * WN + b), 0, g, i);
+  }
   for (int kt = 0; kt < nk; kt++) {
     const int buf = kt & 1;
     const bf16* Ab = As + buf * TA::ELEMS;
     const bf16* Bb = Bs + buf * TB::ELEMS;
+    const bf16* An = As + (buf ^ 1) * TA::ELEMS;
+    const bf16* Bn = Bs + (buf ^ 1) * TB::ELEMS;
     const int kt2 = min(kt + 2, nk - 1);   // past the end: a harmless re-load, and a write nobody reads
-    bf16x8 af[2][WM], bfr[2][WN];
-#pragma unroll
-    for (int a = 0; a < WM; a++) af[0][a] = TA::frag(Ab, 32 * (wm * WM + a), 0, g, i);
-#pragma unroll
-    for (int b = 0; b < WN; b++) bfr[0][b] = TB::frag(Bb, 32 * (wn * WN + b), 0, g, i);
     GEMM_FENCE();
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
@@ -220,25 +230,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
         if (ks + 1 < KSTEPS) {
           af[nxt][a] = TA::frag(Ab, 32 * (wm * WM + a), ks + 1, g, i);
           if (a < WN) bfr[nxt][a] = TB::frag(Bb, 32 * (wn * WN + a), ks + 1, g, i);
+          const int gi = ks * WM + a;
+#pragma unroll
+          for (int m = gi * MOVES / GROUPS; m < (gi + 1) * MOVES / GROUPS; m++) {
+            if (m % 2 == 0) { sstore_a(buf ^ 1, m / 2); gload_a(kt2, m / 2); }
+            else { sstore_b(buf ^ 1, m / 2); gload_b(kt2, m / 2); }
+          }
+        } else {
+          if (a == 0) __syncthreads();
+          // first fragments of the next slab (KSTEPS is even: they land in set 0)
+          af[nxt][a] = TA::frag(An, 32 * (wm * WM + a), 0, g, i);
+          if (a < WN) bfr[nxt][a] = TB::frag(Bn, 32 * (wn * WN + a), 0, g, i);
         }
-        // chunks [ks * C / KSTEPS, (ks + 1) * C / KSTEPS) of both operands, spread over the WM groups of MFMAs
-#pragma unroll
-        for (int j = ks * (CA / KSTEPS); j < (ks + 1) * (CA / KSTEPS); j++)
-          if ((j - ks * (CA / KSTEPS)) * WM / (CA / KSTEPS) == a) {
-            sstore_a(buf ^ 1, j);
-            gload_a(kt2, j);
-          }
-#pragma unroll
-        for (int j = ks * (CB / KSTEPS); j < (ks + 1) * (CB / KSTEPS); j++)
-          if ((j - ks * (CB / KSTEPS)) * WM / (CB / KSTEPS) == a) {
-            sstore_b(buf ^ 1, j);
-            gload_b(kt2, j);
-          }
         GEMM_FENCE();
       }
     }
-    __syncthreads();
   }
+  __syncthreads();   // the epilogue reuses the operand buffers
 
   // Epilogue.  Lane (g, i) holds column m = i and rows n = 8*(r/4) + 4g + r%4 of each 32 x 32 tile,
   // i.e. 8-byte pieces of 32 different rows of C.  Unless C is accumulated into, the tiles go
