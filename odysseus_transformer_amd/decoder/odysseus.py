@@ -215,19 +215,22 @@ class LlamaMLPZeRO(nn.Module):
         if act != "silu":
             raise NotImplementedError(f"hidden_act={act!r}: only the SiLU gate of Llama is implemented")
         self.act_fn = torch.nn.functional.silu  # kept as an attribute for introspection; the fused kernel applies it
+        # SwiGLU (and its backward) inside the products' epilogues; False keeps one kernel per step
+        self.fuse_elementwise = True
 
     def forward(self, x, residual=None):
         """`residual` (an extension: the reference's module takes x only) makes the result
         residual + mlp(x) with every elementwise step fused into the products' epilogues."""
         if getattr(self.config, "pretraining_tp", 1) > 1:
             raise NotImplementedError("pretraining_tp > 1 is not supported yet.")
-        if residual is not None:
-            w1, w2 = self.gate_up_proj.weight, self.down_proj.weight
-            if (get_model_parallel_world_size() == 1 and self.gate_up_proj.bias is None and self.down_proj.bias is None
-                    and x.dtype == residual.dtype == w1.dtype == w2.dtype and not torch.is_autocast_enabled("cuda")):
-                return ops.SwiGLUMLPResidualFunc.apply(x, w1, w2, residual)
-            return residual + self.down_proj(ops.swiglu(self.gate_up_proj(x)))
-        return self.down_proj(ops.swiglu(self.gate_up_proj(x)))
+        w1, w2 = self.gate_up_proj.weight, self.down_proj.weight
+        fusable = (get_model_parallel_world_size() == 1 and self.gate_up_proj.bias is None and self.down_proj.bias is None
+                   and x.dtype == w1.dtype == w2.dtype and (residual is None or residual.dtype == x.dtype)
+                   and not torch.is_autocast_enabled("cuda"))
+        if fusable and self.fuse_elementwise:
+            return ops.SwiGLUMLPResidualFunc.apply(x, w1, w2, residual)
+        y = self.down_proj(ops.swiglu(self.gate_up_proj(x)))
+        return y if residual is None else residual + y
 
 
 class LlamaRMSNorm(nn.Module):
@@ -259,6 +262,7 @@ class OdysseusDecoderLayer(nn.Module):
         eps = getattr(config, "rms_norm_eps", 1e-6)
         self.self_attn = LlamaFlashAttention2TPSP(config, layer_idx)
         self.mlp = LlamaMLPZeRO(config)
+        self.mlp.fuse_elementwise = fused
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
 

@@ -580,19 +580,23 @@ class LinearResidualFunc(torch.autograd.Function):
 
 
 class SwiGLUMLPResidualFunc(torch.autograd.Function):
-    """residual + down(silu(gate) * up) with gate_up = x Wgu^T, every elementwise step inside a product's
-    epilogue: SwiGLU in the gate_up product, the residual add in the down product, the SwiGLU backward
-    in the down product's input gradient (decoder/odysseus.py:293-295 and the add at decoder/ring.py:86)."""
+    """[residual +] down(silu(gate) * up) with gate_up = x Wgu^T, every elementwise step inside a product's
+    epilogue: SwiGLU in the gate_up product, the residual add (when a residual is given) in the down
+    product, the SwiGLU backward in the down product's input gradient (decoder/odysseus.py:293-295 and
+    the add at decoder/ring.py:86)."""
 
     @staticmethod
     def forward(ctx, x, w_gate_up, w_down, residual):
         x2 = x.reshape(-1, x.shape[-1])
         x2 = x2 if x2.stride(1) == 1 else x2.contiguous()
         gate_up, h = linear_swiglu(x2, w_gate_up)
-        y = linear_residual(h, w_down, residual.reshape(-1, residual.shape[-1]))
+        if residual is not None:
+            y = linear_residual(h, w_down, residual.reshape(-1, residual.shape[-1]))
+        else:
+            y = gemm(GEMM_NT, h, w_down)
         ctx.save_for_backward(x2, w_gate_up, w_down, gate_up, h)
-        ctx.x_shape = x.shape
-        return y.view(residual.shape)
+        ctx.x_shape, ctx.has_residual = x.shape, residual is not None
+        return y.view(*x.shape[:-1], w_down.shape[0])
 
     @staticmethod
     def backward(ctx, dy):
@@ -603,7 +607,7 @@ class SwiGLUMLPResidualFunc(torch.autograd.Function):
         dgu = linear_dgrad_swiglu(dy2, w_down, gate_up)
         dx = gemm(GEMM_NN, dgu, w_gate_up).view(ctx.x_shape)
         dw_gate_up = gemm(GEMM_TN, dgu, x2)
-        return dx, dw_gate_up, dw_down, dy
+        return dx, dw_gate_up, dw_down, dy if ctx.has_residual else None
 
 
 def rmsnorm(x, weight, eps: float = 1e-6):
