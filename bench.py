@@ -11,6 +11,8 @@ inputs, already resident in HBM).  `value` is the algorithmic TFLOP/s of that st
   kernels       the same for every attention kernel of the step
   step_ms       median / min / max of the K timed steps (HIP events around each step)
   mfma_sustained  what a loop of nothing but MFMAs sustains with constant and with random operands
+  tile_cost_ladder  a synthetic kernel of the forward kernel's shape with the ingredients of a tile added one at a
+                time (vector work, LDS operand reads, direct loads), ns per 64-key turn, beside the forward kernel
   configs       the other attention configurations (L = 131072; GQA 4:1 at L = 65536; the ring
                 step over 8 key blocks of 16384): ms, TFLOP/s, % of peak, forward / backward split
   layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs with
@@ -128,6 +130,41 @@ def mfma_sustained(_lib, dev):
         e1.record()
         torch.cuda.synchronize()
         res[name + "_tflops"] = round(blocks * 4 * iters * 16 * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+    return res
+
+
+def tile_cost_ladder(_lib, dev, fwd_ms):
+    """What the ingredients of an attention tile cost on top of its MFMAs, measured with a synthetic kernel that has
+    the forward kernel's shape (8 wavefronts, two per SIMD, one workgroup per CU, a barrier per 64-key turn, 32 MFMAs
+    per wavefront and turn) and adds them one at a time -- and the forward kernel itself in the same unit."""
+    import torch
+    blocks, turns = 1024, 2000                   # 4 workgroups per CU in sequence; ~10 ms per rung
+    sink = torch.empty(blocks * 512, dtype=torch.float32, device=dev)
+    g = torch.Generator().manual_seed(7)
+    ops_ = torch.randn(1 << 19, generator=g).to(torch.bfloat16).to(dev)
+    src = torch.randn(32 << 20, generator=g).to(torch.bfloat16).to(dev)     # 64 MiB
+    st = torch.cuda.current_stream().cuda_stream
+    rungs = (("mfma_only", 0), ("plus_vector_work", 1), ("plus_lds_operand_reads", 3), ("plus_direct_loads_only", 5),
+             ("plus_lds_reads_and_direct_loads", 7))
+    res = {}
+    for name, what in rungs:
+        best = None
+        for rep in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.call("ody_pipeline_probe", ops_.data_ptr(), src.data_ptr(), sink.data_ptr(), blocks, turns, what, st)
+            e1.record()
+            torch.cuda.synchronize()
+            if rep:
+                best = e0.elapsed_time(e1) if best is None else min(best, e0.elapsed_time(e1))
+        res[name] = {"ns_per_turn": round(best * 1e6 / (blocks / 256 * turns), 1),
+                     "tflops": round(blocks * 8 * turns * 32 * 32768.0 / (best * 1e-3) / 1e12, 1)}
+    # the forward kernel: 64 MFMAs per SIMD and turn as well; turns = executed MFMAs / (1024 SIMDs * 64)
+    nqb = L // 256
+    tiles = sum(min(L // 64, (qb * 256 + 255) // 64 + 1) for qb in range(nqb)) * H     # 64-key tiles x 256-query blocks
+    mfmas = (tiles * 8 - nqb * H * 12) * 32        # 12 (wavefront, tile) pairs of a diagonal block lie above the diagonal
+    res["attn_fwd_w8"] = {"ns_per_turn": round(fwd_ms * 1e6 / (mfmas / (1024 * 64)), 1),
+                          "tflops_executed": round(mfmas * 32768.0 / (fwd_ms * 1e-3) / 1e12, 1)}
     return res
 
 
@@ -304,6 +341,7 @@ def main():
     out["mfma_sustained"] = mfma_sustained(_lib, dev)
     # boxes differ by ~10 % in what they sustain at the power limit; this ratio does not
     out["value_over_mfma_sustained_random"] = round(value / out["mfma_sustained"]["random_operands_tflops"], 3)
+    out["tile_cost_ladder"] = tile_cost_ladder(_lib, dev, kernels["attn_fwd_w8"]["avg_ms"])
     if a.power:
         out["power"] = power_under_load(_lib, ops, dev, step)
     del qkv, q, k, v, do, dqkv

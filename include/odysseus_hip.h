@@ -69,6 +69,18 @@ int ody_profile_collect(char* out, size_t cap);
  */
 int ody_mfma_probe(const void* operands, float* sink, int blocks, int iters, void* stream);
 
+/* Measurement aid (no counterpart in the reference): what each ingredient of an attention tile costs on
+ * top of the bare MFMAs.  Workgroups of 8 wavefronts (two per SIMD, 96 KB of LDS: one per CU), a barrier
+ * per turn, 32 MFMAs per wavefront and turn; `what` adds the vector work of a 32 x 64 score tile
+ * (ODY_PROBE_VECTOR), the MFMA A operands read from LDS (ODY_PROBE_LDS_READS) and 32 KB of direct
+ * global->LDS loads per turn and workgroup, two turns ahead (ODY_PROBE_DIRECT_LOADS, from the 64 MiB at
+ * stream_src).  Built combinations: 0, 1, 3, 5, 7.  operands: at least 1 MiB of bf16; sink: blocks * 512
+ * floats.  FLOP: blocks * 8 * turns * 32 * 32768.
+ */
+enum ody_probe_parts { ODY_PROBE_VECTOR = 1, ODY_PROBE_LDS_READS = 2, ODY_PROBE_DIRECT_LOADS = 4 };
+int ody_pipeline_probe(const void* operands, const void* stream_src, float* sink, int blocks, int turns, int what,
+                       void* stream);
+
 /* ---- attention ---------------------------------------------------------
  * Replaces flash_attn_func(q, k, v, dropout_p=0, softmax_scale, causal) as
  * reached from decoder/odysseus.py:256-263 (via HF _flash_attention_forward),

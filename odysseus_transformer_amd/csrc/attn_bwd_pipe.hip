@@ -196,9 +196,10 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
     __syncthreads();
     const bf16* st = ring + (t % 3) * STAGE;
     const bool dead = p.causal && t * BN > wq0 + 32 * QT - 1 + p.off;   // every key of the tile is after this wavefront's queries
+    if (!dead) tile(st, t, t >= n_full);
+    // the loads go last: issuing them costs this wavefront time, and here it would otherwise wait at the barrier
     if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 0);
     if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 1);
-    if (!dead) tile(st, t, t >= n_full);
   }
 
 #pragma unroll

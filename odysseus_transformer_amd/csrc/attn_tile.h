@@ -126,14 +126,18 @@ __device__ __forceinline__ int fresh_lane() {
 // vector phase -- and the matrix pipe idles half of the time.  Raising the priority of the
 // first wavefront to arrive on each SIMD breaks the symmetry: it runs ahead, and the other
 // one fills the matrix pipe while the first is in its vector phase.
-__device__ __forceinline__ void simd_stagger(int tid) {
+// Order of arrival of this wavefront among those of its workgroup on the same SIMD (0, 1, ...).
+__device__ __forceinline__ int simd_rank(int tid) {
   __shared__ int simd_count[4];
   if (tid < 4) simd_count[tid] = 0;
   __syncthreads();
   const int simd = __builtin_amdgcn_s_getreg((1 << 11) | (4 << 6) | 4) & 3;   // HW_ID.SIMD_ID
   int rank = 0;
   if ((tid & 63) == 0) rank = atomicAdd(&simd_count[simd], 1);
-  if (__builtin_amdgcn_readfirstlane(rank) == 0) __builtin_amdgcn_s_setprio(2);
+  return __builtin_amdgcn_readfirstlane(rank);
+}
+__device__ __forceinline__ void simd_stagger(int tid) {
+  if (simd_rank(tid) == 0) __builtin_amdgcn_s_setprio(2);
 }
 
 // Swap of the two wavefront halves through v_permlane32_swap: returns, in every lane,

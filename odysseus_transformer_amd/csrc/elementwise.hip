@@ -94,13 +94,16 @@ __global__ __launch_bounds__(256) void rmsnorm_fwd_kernel(const T* __restrict__ 
 // ---------------------------------------------------------------------------
 constexpr int RMS_BWD_MAXK = 4;  // column vectors per lane: d <= 256 * N * MAXK
 
-template <typename T>
+// MAXK: column vectors per lane this instance is built for (d <= 256 * N * MAXK).  The raw vectors of the next
+// row are fetched before the current row's sum is reduced, so that a block always has a row of loads in flight.
+template <typename T, int MAXK>
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                           const float* __restrict__ rstd, const T* __restrict__ dy,
                                                           T* __restrict__ dx, float* __restrict__ dw_partial,
                                                           int Trows, int d, int rows_per_block,
                                                           const T* __restrict__ dx_add) {
-  constexpr int N = VecIO<T>::N, MAXK = RMS_BWD_MAXK;
+  constexpr int N = VecIO<T>::N;
+  typedef typename VecIO<T>::vec_t vec_t;
   __shared__ float red[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int nvec = d / N;
@@ -113,7 +116,22 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     for (int e = 0; e < N; e++) acc[k][e] = 0.f, wf[k][e] = 0.f;
     if (vi < nvec) VecIO<T>::load(w + vi * N, wf[k]);
   }
+  vec_t xr[MAXK], dyr[MAXK], ar[MAXK];   // raw vectors of the row in hand
+  auto fetch = [&](int row, vec_t (&xv)[MAXK], vec_t (&dv)[MAXK], vec_t (&av)[MAXK]) {
+#pragma unroll
+    for (int k = 0; k < MAXK; k++) {
+      const int vi = tid + 256 * k;
+      if (vi < nvec) {
+        xv[k] = *reinterpret_cast<const vec_t*>(x + (int64_t)row * d + vi * N);
+        dv[k] = *reinterpret_cast<const vec_t*>(dy + (int64_t)row * d + vi * N);
+        if (dx_add) av[k] = *reinterpret_cast<const vec_t*>(dx_add + (int64_t)row * d + vi * N);
+      }
+    }
+  };
+  if (r0 < r1) fetch(r0, xr, dyr, ar);
   for (int row = r0; row < r1; row++) {
+    vec_t xn[MAXK], dyn[MAXK], an[MAXK];
+    if (row + 1 < r1) fetch(row + 1, xn, dyn, an);
     const float rs = rstd[row];
     float xh[MAXK][N], gv[MAXK][N];
     float part = 0.f;
@@ -121,15 +139,13 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     for (int k = 0; k < MAXK; k++) {
       const int vi = tid + 256 * k;
       if (vi < nvec) {
-        float dyv[N];
-        VecIO<T>::load(x + (int64_t)row * d + vi * N, xh[k]);
-        VecIO<T>::load(dy + (int64_t)row * d + vi * N, dyv);
 #pragma unroll
         for (int e = 0; e < N; e++) {
-          xh[k][e] *= rs;
-          gv[k][e] = dyv[e] * wf[k][e];
+          const float dyv = (float)dyr[k][e];
+          xh[k][e] = (float)xr[k][e] * rs;
+          gv[k][e] = dyv * wf[k][e];
           part = fmaf(gv[k][e], xh[k][e], part);
-          acc[k][e] = fmaf(dyv[e], xh[k][e], acc[k][e]);
+          acc[k][e] = fmaf(dyv, xh[k][e], acc[k][e]);
         }
       }
     }
@@ -142,14 +158,18 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
     for (int k = 0; k < MAXK; k++) {
       const int vi = tid + 256 * k;
       if (vi < nvec) {
-        float o[N], add[N];
+        float o[N];
 #pragma unroll
-        for (int e = 0; e < N; e++) add[e] = 0.f;
-        if (dx_add) VecIO<T>::load(dx_add + (int64_t)row * d + vi * N, add);   // gradient arriving over the residual path
-#pragma unroll
-        for (int e = 0; e < N; e++) o[e] = add[e] + rs * (gv[k][e] - xh[k][e] * c);
+        for (int e = 0; e < N; e++) {
+          const float add = dx_add ? (float)ar[k][e] : 0.f;   // gradient arriving over the residual path
+          o[e] = add + rs * (gv[k][e] - xh[k][e] * c);
+        }
         VecIO<T>::store(dx + (int64_t)row * d + vi * N, o);
       }
+    }
+    if (row + 1 < r1) {
+#pragma unroll
+      for (int k = 0; k < MAXK; k++) xr[k] = xn[k], dyr[k] = dyn[k], ar[k] = an[k];
     }
   }
 #pragma unroll
@@ -160,6 +180,19 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const T* __restrict__ 
       for (int e = 0; e < N; e++) dw_partial[(int64_t)blockIdx.x * d + vi * N + e] = acc[k][e];
     }
   }
+}
+
+template <typename T>
+void launch_rmsnorm_bwd(hipStream_t st, int nblocks, const void* x, const void* w, const float* rstd, const void* dy,
+                        void* dx, float* dw_partial, int T_, int d, int rpb, const void* dx_add) {
+  const int nvec = d / VecIO<T>::N;
+#define ODY_RMS_BWD(K)                                                                                              \
+  ODY_LAUNCH("rmsnorm_bwd", st, (rmsnorm_bwd_kernel<T, K>), dim3(nblocks), dim3(256), 0, (const T*)x, (const T*)w, rstd, \
+             (const T*)dy, (T*)dx, dw_partial, T_, d, rpb, (const T*)dx_add)
+  if (nvec <= 256) ODY_RMS_BWD(1);
+  else if (nvec <= 512) ODY_RMS_BWD(2);
+  else ODY_RMS_BWD(4);
+#undef ODY_RMS_BWD
 }
 
 // out[c] = sum_r partial[r][c].  A block owns 16 columns (64-byte row pieces) and splits the rows
@@ -362,13 +395,8 @@ extern "C" int ody_rmsnorm_bwd(const void* x, const void* w, const float* rstd, 
   const int nparts = ody_rmsnorm_bwd_partials(T);
   const int rpb = (T + nparts - 1) / nparts;
   const int nblocks = (T + rpb - 1) / rpb;  // <= nparts; rows of dw_partial beyond nblocks are not written
-  ODY_BY_DTYPE(dtype,
-               ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<bf16>, dim3(nblocks), dim3(256), 0, (const bf16*)x,
-                                  (const bf16*)w, rstd, (const bf16*)dy, (bf16*)dx, dw_partial, T, d, rpb,
-                                  (const bf16*)dx_add),
-               ODY_LAUNCH("rmsnorm_bwd", st, rmsnorm_bwd_kernel<float>, dim3(nblocks), dim3(256), 0, (const float*)x,
-                                  (const float*)w, rstd, (const float*)dy, (float*)dx, dw_partial, T, d, rpb,
-                                  (const float*)dx_add));
+  ODY_BY_DTYPE(dtype, launch_rmsnorm_bwd<bf16>(st, nblocks, x, w, rstd, dy, dx, dw_partial, T, d, rpb, dx_add),
+               launch_rmsnorm_bwd<float>(st, nblocks, x, w, rstd, dy, dx, dw_partial, T, d, rpb, dx_add));
   int rc = ody_check_launch("rmsnorm_bwd");
   if (rc || !dw) return rc;
   ODY_BY_DTYPE(dtype,
