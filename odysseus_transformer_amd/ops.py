@@ -481,6 +481,87 @@ def ring_blocks_attn(q, k_blocks, v_blocks, causal_block: Optional[int] = 0, sof
     return RingBlocksAttnFunc.apply(q, cb, softmax_scale, *k_blocks, *v_blocks)
 
 
+class ZigzagRingRankAttnFunc(torch.autograd.Function):
+    """One rank's compute of zigzag ring attention (the routine decoder/ring.py:30-37 of the reference calls,
+    ring_flash_attn's zigzag_ring_flash_attn_func: the sequence is cut into 2N chunks and rank r holds chunks r and
+    2N-1-r, see utils/apply_seq_parallel.py:93-99).  The K/V blocks a rank receives over the ring are arguments
+    here: block s is the local K/V of rank (r - s) mod N.
+
+        step 0           local queries x local keys, causal (chunk r precedes chunk 2N-1-r)
+        source rank < r  all local queries x the FIRST chunk of the block, fully visible
+        source rank > r  the queries of the SECOND local chunk x the whole block, fully visible
+
+    Every step's (out, lse) is merged into fp32 running pairs (one per local chunk); backward runs the per-step
+    flash backward with the final out / lse, a running fp32 dq, and returns each block's dK / dV (zero in the
+    half a step did not read), which the ring would send on with the block.
+
+    apply(q, rank, world_size, softmax_scale, *k_blocks, *v_blocks) -> (out, lse)."""
+
+    @staticmethod
+    def _steps(rank, world):
+        """[(query chunk range, key chunk range, causal)] in units of chunks of the local sequence (0..2)."""
+        steps = [((0, 2), (0, 2), True)]
+        for s in range(1, world):
+            src = (rank - s) % world
+            steps.append(((0, 2), (0, 1), False) if src < rank else ((1, 2), (0, 2), False))
+        return steps
+
+    @staticmethod
+    def forward(ctx, q, rank, world, softmax_scale, *kv):
+        if len(kv) != 2 * world:
+            raise ValueError(f"{world} key and {world} value blocks expected, got {len(kv)} tensors")
+        ks, vs = kv[:world], kv[world:]
+        B, L2, H, D = q.shape
+        if L2 % 2:
+            raise ValueError(f"the local sequence holds two chunks of equal length, got {L2} tokens")
+        c = L2 // 2
+        for t in kv:
+            if t.shape[1] != L2:
+                raise ValueError(f"every block holds two chunks of {c} tokens, got {tuple(t.shape)}")
+        acc = [torch.zeros((B, c, H, D), dtype=torch.float32, device=q.device) for _ in range(2)]
+        lse = [torch.full((B, H, c), float("-inf"), dtype=torch.float32, device=q.device) for _ in range(2)]
+        for s, ((q0, q1), (k0, k1), causal) in enumerate(ZigzagRingRankAttnFunc._steps(rank, world)):
+            ob, lb = attn_fwd(q[:, q0 * c:q1 * c], ks[s][:, k0 * c:k1 * c], vs[s][:, k0 * c:k1 * c], causal=causal,
+                              scale=softmax_scale)
+            for i, ch in enumerate(range(q0, q1)):
+                lb_ch = lb if q1 - q0 == 1 else lb[:, :, i * c:(i + 1) * c].contiguous()
+                lse_merge_(acc[ch], lse[ch], ob[:, i * c:(i + 1) * c], lb_ch)
+        out = torch.cat([cast_from_f32(a, q.dtype) for a in acc], dim=1)
+        lse_full = torch.cat(lse, dim=2)
+        ctx.save_for_backward(q, out, lse_full, *kv)
+        ctx.rank, ctx.world, ctx.softmax_scale = rank, world, softmax_scale
+        ctx.mark_non_differentiable(lse_full)
+        return out, lse_full
+
+    @staticmethod
+    def backward(ctx, dout, _dlse):
+        q, out, lse, *kv = ctx.saved_tensors
+        world = ctx.world
+        ks, vs = kv[:world], kv[world:]
+        c = q.shape[1] // 2
+        if dout.stride(3) != 1:
+            dout = dout.contiguous()
+        dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+        lse_b = lse[:, :, c:].contiguous()
+        ws = attn_bwd_workspace(q, ks[0])
+        dks = [torch.zeros_like(k) for k in ks]
+        dvs = [torch.zeros_like(v) for v in vs]
+        prev = None
+        for s, ((q0, q1), (k0, k1), causal) in enumerate(ZigzagRingRankAttnFunc._steps(ctx.rank, world)):
+            qs, kr = slice(q0 * c, q1 * c), slice(k0 * c, k1 * c)
+            kind = (q0, q1, k0, k1)
+            attn_bwd(q[:, qs], ks[s][:, kr], vs[s][:, kr], out[:, qs], lse if q1 - q0 == 2 else lse_b, dout[:, qs],
+                     causal=causal, scale=ctx.softmax_scale, dq=dq[:, qs], dk=dks[s][:, kr], dv=dvs[s][:, kr],
+                     accumulate_dq=(s > 0), workspace=ws, reuse_query_side=(kind == prev))
+            prev = kind
+        return (cast_from_f32(dq, q.dtype), None, None, None, *dks, *dvs)
+
+
+def zigzag_ring_rank_attn(q, k_blocks, v_blocks, rank: int, world_size: int, softmax_scale: Optional[float] = None):
+    """Functional form of ZigzagRingRankAttnFunc: (out, lse) of rank `rank`'s two chunks."""
+    return ZigzagRingRankAttnFunc.apply(q, int(rank), int(world_size), softmax_scale, *k_blocks, *v_blocks)
+
+
 def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[float] = None, causal: bool = False,
                     return_lse: bool = False):
     """Signature of the routine the reference reaches at decoder/odysseus.py:256-263.

@@ -8,14 +8,16 @@ set-up and at every step, `loss.backward(loss)`, AdamW, and one line
 "<mode> <L/1024>K <world> Time taken: <s> seconds" at the end (train.py:167-235).  The model is the
 16-layer GQA 32/8 configuration of train.py:66-76, randomly initialised (no checkpoint can be
 fetched here; `--model` takes a local directory only), patched with
-apply_odysseus_attn_patch_llama / apply_tpsp_attn_patch_llama, with the loss from the fused
-cross-entropy kernel.
+apply_odysseus_attn_patch_llama / apply_tpsp_attn_patch_llama (or, for the ulysses, ring and dp modes,
+with the host's attention routed to the HIP flash attention: with one rank their all-to-alls and block
+exchanges are the identity), with the loss from the fused cross-entropy kernel.
 
 What differs from the reference and why: one process, one GPU, no FSDP wrapping (its world-size-1
 branch skips it too, train.py:118); `--native-host-modules` (default on) also routes the host
-model's RMSNorms and lm_head through the HIP library, so that the step runs on this library's
-kernels except for the embedding lookup, the residual adds of the host decoder layer and the
-optimizer; switch it off to keep every host module as transformers ships it.
+model's RMSNorms, lm_head and whatever bias-free projections the patch left in its layers through
+the HIP library, so that the step runs on this library's kernels except for the embedding lookup,
+the residual adds (and, in the ulysses / ring / dp modes, the rotary embedding and SiLU-multiply)
+of the host decoder layer and the optimizer; switch it off to keep every host module as transformers ships it.
 """
 from __future__ import annotations
 
@@ -54,6 +56,11 @@ def use_native_host_modules(model) -> None:
     for layer in model.model.layers:
         layer.input_layernorm = native_norm(layer.input_layernorm)
         layer.post_attention_layernorm = native_norm(layer.post_attention_layernorm)
+        # the host's own projections (the modes that keep its attention / MLP modules: ulysses, ring, dp)
+        for parent in (layer.self_attn, layer.mlp):
+            for name, child in list(parent.named_children()):
+                if type(child) is nn.Linear and child.bias is None:
+                    setattr(parent, name, NativeLinear(child))
     model.model.norm = native_norm(model.model.norm)
     model.lm_head = NativeLinear(model.lm_head)
 
@@ -112,9 +119,15 @@ def main(args) -> dict:
     elif args.parallel_mode == "tpsp":
         with torch.device(dev):
             apply_tpsp_attn_patch_llama(model)
-    else:
-        raise SystemExit(f"parallel_mode {args.parallel_mode!r}: this build has the odysseus and tpsp modules "
-                         "(ulysses, ring and dp are collective choreography, which is out of its scope)")
+    elif args.parallel_mode == "ulysses":
+        from .decoder.ulysses import apply_ulysses_attn_monkey_patch_llama
+        apply_ulysses_attn_monkey_patch_llama(model)
+    elif args.parallel_mode == "ring":
+        from .decoder.ring import apply_zigzag_ring_attn_monkey_patch_llama
+        apply_zigzag_ring_attn_monkey_patch_llama(model)
+    else:   # dp: the host model as it is; its flash-attention call lands on the HIP kernel (flash_attn is not installed)
+        from .decoder.ulysses import install_hip_flash_attention, hip_ulysses_attention_forward
+        install_hip_flash_attention(hip_ulysses_attention_forward, model)
     model = model.to(dev)
     from .utils.linear_zero3 import LinearZeRO3
     with torch.no_grad():     # LinearZeRO3 leaves its weight uninitialised, as the reference does: give it finite values

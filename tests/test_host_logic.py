@@ -275,3 +275,51 @@ def test_tpsp_mlp_surface():
     assert tuple(m.w1w3.weight.shape) == (48, 64) and tuple(m.w2.weight.shape) == (64, 24)
     with pytest.raises(AssertionError, match="Pretraining TP"):
         LlamaMLPTPSP(_cfg(pretraining_tp=2))(torch.zeros(1, 4, 64))
+
+
+def test_zigzag_step_table():
+    """Which part of a received block a rank uses (zigzag ring): a source rank before it contributes its first
+    chunk to all local queries, a source rank after it is seen by the second local chunk only."""
+    from odysseus_transformer_amd.ops import ZigzagRingRankAttnFunc as Z
+    assert Z._steps(0, 1) == [((0, 2), (0, 2), True)]
+    # rank 1 of 4 receives the blocks of ranks 1, 0, 3, 2
+    assert Z._steps(1, 4) == [((0, 2), (0, 2), True), ((0, 2), (0, 1), False), ((1, 2), (0, 2), False),
+                              ((1, 2), (0, 2), False)]
+    # brute force over token positions: the steps of every rank cover each (query, key <= query) chunk pair once
+    for world in (1, 2, 3, 5):
+        seen = {}
+        for r in range(world):
+            mine = (r, 2 * world - 1 - r)
+            for s, ((q0, q1), (k0, k1), causal) in enumerate(Z._steps(r, world)):
+                src = (r - s) % world
+                theirs = (src, 2 * world - 1 - src)
+                for qi in range(q0, q1):
+                    for ki in range(k0, k1):
+                        qc, kc = mine[qi], theirs[ki]
+                        if causal and kc > qc:
+                            continue            # masked inside the causal step
+                        assert kc <= qc, (world, r, s, qc, kc)
+                        seen[(qc, kc)] = seen.get((qc, kc), 0) + 1
+        assert all(n == 1 for n in seen.values())
+        assert len(seen) == (2 * world) * (2 * world + 1) // 2
+
+
+def test_ring_and_ulysses_refuse_a_larger_world():
+    import pytest as _pytest
+    from odysseus_transformer_amd import parallel_state
+    from odysseus_transformer_amd.decoder.ring import zigzag_ring_flash_attn_func
+    from odysseus_transformer_amd.decoder.ulysses import ulysses_attn
+    parallel_state.initialize_model_parallel(2, 0)
+    try:
+        with _pytest.raises(NotImplementedError):
+            zigzag_ring_flash_attn_func(None, None, None, 0.0, None, causal=True)
+        with _pytest.raises(NotImplementedError):
+            ulysses_attn(None, None, None)
+    finally:
+        parallel_state.destroy_model_parallel()
+
+
+def test_train_script_accepts_every_mode_of_the_reference():
+    from odysseus_transformer_amd.train import parse_args
+    for mode in ("odysseus", "ulysses", "dp", "tpsp", "ring"):
+        assert parse_args(["--parallel_mode", mode]).parallel_mode == mode
