@@ -478,8 +478,9 @@ def layer_end_to_end(_lib, rn, dev, pieces):
             "layer_tokens_per_s_per_gpu": round(T_MLP / (med * 1e-3), 1),
             "sum_of_pieces_tokens_per_s_per_gpu": pieces["layer_tokens_per_s_per_gpu"],
             "scratch": "attention, split-K and norm workspaces drawn from the GlobalMemoryBuffer arena",
-            "fusions": "SwiGLU forward / backward and the MLP's residual add run in GEMM epilogues, the gradient sum at the "
-                       "fork of the residual stream inside the RMSNorm backward"}
+            "fusions": "SwiGLU forward / backward, both residual adds and the rotary embedding run in GEMM epilogues, the "
+                       "rotary backward in the attention backward's epilogues, the gradient sum at the fork of the "
+                       "residual stream inside the RMSNorm backward"}
 
 
 def layer_share(_lib, ops, rn, dev, attn_sec):
@@ -539,6 +540,18 @@ def layer_share(_lib, ops, rn, dev, attn_sec):
     rope_bytes = 2 * L * (H + HKV) * D * e
     t_attn_half += 2 * membound("rope", lambda: ops.rope_(qkv, H + HKV), rope_bytes)
     del qkv
+    # the same rotation inside the QKV projection's epilogue (what the modules run): table + fused product, by kernel events
+    xq, wq = rn((L, D_MODEL), 8), rn(((H + 2 * HKV) * D, D_MODEL), 9, std=0.02)
+    _lib.profile_enable(True)
+    _lib.profile_collect()
+    for _ in range(10):
+        ops.linear_rope(xq, wq, ops.rope_table(None, L, D, 10000.0, device=dev), H + HKV, D)
+    torch.cuda.synchronize()
+    prof = _lib.profile_collect()
+    _lib.profile_enable(False)
+    res["qkv_proj_with_rope"] = {"kernels_ms": {k: round(v[1] / 10, 4) for k, v in sorted(prof.items())},
+                                 "fwd_tflops": round(2.0 * L * (H + 2 * HKV) * D * D_MODEL / (prof["gemm_bf16_nt_rope"][1] / 10 * 1e-3) / 1e12, 1)}
+    del xq, wq
 
     t_mlp_half = gemm3("gate_up_proj", T_MLP, 2 * I_MLP, D_MODEL)
     t_mlp_half += gemm3("down_proj", T_MLP, D_MODEL, I_MLP)

@@ -274,6 +274,40 @@ int ody_rope(void* x, const int64_t* position_ids, const float* inv_freq, int B,
              int D, int64_t sx_b, int64_t sx_l, int64_t sx_h, float base, int inverse,
              int dtype, void* stream);
 
+/* The same rotary embedding fused into its neighbours (bf16, head_dim 128), so that no pass over the packed
+ * projection is left: the rotation of q and k (decoder/odysseus.py:210-213) rides in the epilogue of the QKV
+ * projection (utils/linear_tpsp.py:173), and its backward in the epilogues of the attention backward.
+ *
+ * ody_rope_table   table (rows, D) bf16: table[r][2 j] = cos, table[r][2 j + 1] = sin of position_ids[r] *
+ *                  inv_freq[j], j < D / 2 (NULL position_ids: r; NULL inv_freq: base^(-2j/D)), rounded to bf16 as
+ *                  ody_rope rounds them.  rows = B * L in the order of the projection's rows; contiguous (ld_table = D).
+ * ody_linear_rope  y (M, N) = x (M, K) w (N, K)^T with the first n_rot heads of D columns rotated by the table's row m
+ *                  before the one rounding to bf16 (ody_gemm + ody_rope round twice).  Any shape: products the fused
+ *                  kernel does not take run as the plain product followed by the rotation from the table.
+ * ody_attn_bwd_rope  ody_attn_bwd whose dq and dk leave the kernels rotated back by the negative angle, i.e. as the
+ *                  gradient of the projection before its rotary embedding: rope_table_q holds the rows of the
+ *                  queries (B * Lq, pitch D), rope_table_k those of the keys (B * Lk).  Not with ODY_BWD_ACCUMULATE_DQ
+ *                  or ODY_BWD_DQ_F32.
+ */
+int ody_rope_table(const int64_t* position_ids, const float* inv_freq, int64_t rows, int D, float base,
+                   void* table, void* stream);
+int ody_linear_rope(const void* x, const void* w, const void* table, void* y, int M, int N, int K, int n_rot,
+                    int D, int64_t ldx, int64_t ldw, int64_t ld_table, int64_t ldy, int dtype, void* stream);
+int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                      const void* dout, void* dq, void* dk, void* dv,
+                      int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                      int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                      int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                      int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                      int64_t so_b, int64_t so_l, int64_t so_h,
+                      int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                      int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                      int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                      int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                      float scale, int causal, int flags, int dtype,
+                      void* workspace, size_t workspace_bytes, void* stream,
+                      const void* rope_table_q, const void* rope_table_k);
+
 /* ---- cross-entropy over the vocabulary --------------------------------------
  * flash_attn.losses.cross_entropy.CrossEntropyLoss(inplace_backward=True) as the training loop
  * uses it (train.py:8,173,212-214): softmax cross-entropy of logits (T, V) (row stride ld,

@@ -134,6 +134,72 @@ extern "C" size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, in
   return n;
 }
 
+namespace {
+int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
+                  const void* q, const void* k, const void* v, const void* out, const float* lse,
+                  const void* dout, void* dq, void* dk, void* dv,
+                  int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                  int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                  int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                  int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                  int64_t so_b, int64_t so_l, int64_t so_h,
+                  int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                  int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                  int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                  int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                  float scale, int causal, int flags, int dtype,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_common(who, B, Lq, Lk, Hq, Hkv, D, dtype);
+  if (rc) return rc;
+  ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE)) == 0, ODY_ERR_UNSUPPORTED,
+              "%s: unknown flag bits in %d", who, flags);
+  AttnParams p{};
+  p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
+  p.dout = dout; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.causal = causal ? 1 : 0; p.off = Lk - Lq; p.accumulate_dq = (flags & ODY_BWD_ACCUMULATE_DQ) ? 1 : 0;
+  p.dq_f32 = (flags & ODY_BWD_DQ_F32) || dtype == ODY_F32 ? 1 : 0;
+  p.reuse_query_side = (flags & ODY_BWD_REUSE_QUERY_SIDE) ? 1 : 0;
+  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
+  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
+  p.sdo = {sdo_b, sdo_l, sdo_h}; p.sdq = {sdq_b, sdq_l, sdq_h}; p.sdk = {sdk_b, sdk_l, sdk_h};
+  p.sdv = {sdv_b, sdv_l, sdv_h};
+  const bool vec = true;
+  if ((rc = check_tensor(who, "q", q, p.sq, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "k", k, p.sk, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "out", out, p.so, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dq", dq, p.sdq, p.dq_f32 ? ODY_F32 : dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dk", dk, p.sdk, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "dv", dv, p.sdv, dtype, vec))) return rc;
+  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "%s: lse is NULL", who);
+  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "%s: scale must be positive", who);
+  ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "%s: workspace is NULL", who);
+  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype), ODY_ERR_WORKSPACE,
+              "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
+              ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype));
+  ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
+              "%s: workspace must be 256-byte aligned", who);
+  if (rope_q || rope_k) {
+    ODY_REQUIRE(rope_q && rope_k, ODY_ERR_NULL, "%s: both tables or none", who);
+    ODY_REQUIRE(dtype == ODY_BF16 && D == 128, ODY_ERR_UNSUPPORTED, "%s: the rotary tables need bf16 and head_dim 128", who);
+    ODY_REQUIRE(!p.dq_f32 && !p.accumulate_dq, ODY_ERR_UNSUPPORTED,
+                "%s: the rotary tables cannot be combined with an accumulated or fp32 dq", who);
+    ODY_REQUIRE(ody_aligned16(rope_q) && ody_aligned16(rope_k), ODY_ERR_MISALIGNED, "%s: tables must be 16-byte aligned", who);
+    p.rope_q = static_cast<const bf16*>(rope_q);
+    p.rope_k = static_cast<const bf16*>(rope_k);
+  }
+  p.delta = static_cast<float*>(workspace);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && D == 128)   // its query-side pre-pass computes delta as well
+    return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
+  if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
+  if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
+  return ody_launch_attn_bwd_f32(p, D, st);
+}
+}  // namespace
+
 extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
                             const void* dout, void* dq, void* dk, void* dv,
                             int B, int Lq, int Lk, int Hq, int Hkv, int D,
@@ -147,44 +213,27 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
                             int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
                             float scale, int causal, int flags, int dtype,
                             void* workspace, size_t workspace_bytes, void* stream) {
-  int rc = check_common("ody_attn_bwd", B, Lq, Lk, Hq, Hkv, D, dtype);
-  if (rc) return rc;
-  ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE)) == 0, ODY_ERR_UNSUPPORTED,
-              "ody_attn_bwd: unknown flag bits in %d", flags);
-  AttnParams p{};
-  p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
-  p.dout = dout; p.dq = dq; p.dk = dk; p.dv = dv;
-  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
-  p.causal = causal ? 1 : 0; p.off = Lk - Lq; p.accumulate_dq = (flags & ODY_BWD_ACCUMULATE_DQ) ? 1 : 0;
-  p.dq_f32 = (flags & ODY_BWD_DQ_F32) || dtype == ODY_F32 ? 1 : 0;
-  p.reuse_query_side = (flags & ODY_BWD_REUSE_QUERY_SIDE) ? 1 : 0;
-  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
-  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
-  p.sdo = {sdo_b, sdo_l, sdo_h}; p.sdq = {sdq_b, sdq_l, sdq_h}; p.sdk = {sdk_b, sdk_l, sdk_h};
-  p.sdv = {sdv_b, sdv_l, sdv_h};
-  const bool vec = true;
-  const char* who = "ody_attn_bwd";
-  if ((rc = check_tensor(who, "q", q, p.sq, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "k", k, p.sk, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "out", out, p.so, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "dout", dout, p.sdo, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "dq", dq, p.sdq, p.dq_f32 ? ODY_F32 : dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "dk", dk, p.sdk, dtype, vec))) return rc;
-  if ((rc = check_tensor(who, "dv", dv, p.sdv, dtype, vec))) return rc;
-  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_bwd: lse is NULL");
-  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_bwd: scale must be positive");
-  ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_bwd: workspace is NULL");
-  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype), ODY_ERR_WORKSPACE,
-              "ody_attn_bwd: workspace of %zu bytes, %zu needed", workspace_bytes,
-              ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype));
-  ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
-              "ody_attn_bwd: workspace must be 256-byte aligned");
-  p.delta = static_cast<float*>(workspace);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == ODY_BF16 && D == 128)   // its query-side pre-pass computes delta as well
-    return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
-  if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
-  if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
-  return ody_launch_attn_bwd_f32(p, D, st);
+  return attn_bwd_impl("ody_attn_bwd", nullptr, nullptr, q, k, v, out, lse, dout, dq, dk, dv, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h,
+                       so_b, so_l, so_h, sdo_b, sdo_l, sdo_h, sdq_b, sdq_l, sdq_h, sdk_b, sdk_l, sdk_h, sdv_b, sdv_l, sdv_h, scale,
+                       causal, flags, dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                            const void* dout, void* dq, void* dk, void* dv,
+                            int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                            int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                            int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                            int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                            int64_t so_b, int64_t so_l, int64_t so_h,
+                            int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                            int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                            int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                            int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                            float scale, int causal, int flags, int dtype,
+                            void* workspace, size_t workspace_bytes, void* stream,
+                            const void* rope_table_q, const void* rope_table_k) {
+  ODY_REQUIRE(rope_table_q && rope_table_k, ODY_ERR_NULL, "ody_attn_bwd_rope: rotary table is NULL");
+  return attn_bwd_impl("ody_attn_bwd_rope", rope_table_q, rope_table_k, q, k, v, out, lse, dout, dq, dk, dv, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h,
+                       so_b, so_l, so_h, sdo_b, sdo_l, sdo_h, sdq_b, sdq_l, sdq_h, sdk_b, sdk_l, sdk_h, sdv_b, sdv_l, sdv_h, scale,
+                       causal, flags, dtype, workspace, workspace_bytes, stream);
 }

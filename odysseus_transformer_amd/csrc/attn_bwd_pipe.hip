@@ -219,6 +219,26 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
           for (int e = 0; e < 4; e++) w[e] += dq[qt][dt][4 * a + e] * p.scale;
           *dst = w;
         }
+    } else if (qi < p.Lq && p.rope_q) {
+      // the gradient of the un-rotated projection: element d < 64 pairs with d + 64, both in this lane
+      bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+      const bf16* trow = p.rope_q + ((int64_t)b * p.Lq + qi) * D;
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          const bf16x8 cs = *reinterpret_cast<const bf16x8*>(trow + 2 * (32 * dt + 8 * a + 4 * g));
+          bf16x4 w1, w2;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+            const float g1 = dq[qt][dt][4 * a + e] * p.scale, g2 = dq[qt][dt + 2][4 * a + e] * p.scale;
+            w1[e] = (bf16)(g1 * c + g2 * sn);
+            w2[e] = (bf16)(g2 * c - g1 * sn);
+          }
+          *reinterpret_cast<bf16x4*>(dqp + 32 * dt + 8 * a + 4 * g) = w1;
+          *reinterpret_cast<bf16x4*>(dqp + 32 * (dt + 2) + 8 * a + 4 * g) = w2;
+        }
     } else if (qi < p.Lq) {
       bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
 #pragma unroll
@@ -441,43 +461,89 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   } else if (key < p.Lk) {
     bf16* dkp = static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l;
     bf16* dvp = static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l;
+    const bf16* trow = p.rope_k ? p.rope_k + ((int64_t)b * p.Lk + key) * D : nullptr;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
       for (int a = 0; a < 4; a++) {
-        bf16x4 wk, wv;
+        bf16x4 wv;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          wk[e] = (bf16)(dk[dt][4 * a + e] * p.scale);
-          wv[e] = (bf16)dv[dt][4 * a + e];
-        }
-        *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = wk;
+        for (int e = 0; e < 4; e++) wv[e] = (bf16)dv[dt][4 * a + e];
         *reinterpret_cast<bf16x4*>(dvp + 32 * dt + 8 * a + 4 * g) = wv;
       }
+    if (trow) {   // dK of the un-rotated projection: element d < 64 pairs with d + 64, both in this lane
+#pragma unroll
+      for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          const bf16x8 cs = *reinterpret_cast<const bf16x8*>(trow + 2 * (32 * dt + 8 * a + 4 * g));
+          bf16x4 w1, w2;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+            const float g1 = dk[dt][4 * a + e] * p.scale, g2 = dk[dt + 2][4 * a + e] * p.scale;
+            w1[e] = (bf16)(g1 * c + g2 * sn);
+            w2[e] = (bf16)(g2 * c - g1 * sn);
+          }
+          *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = w1;
+          *reinterpret_cast<bf16x4*>(dkp + 32 * (dt + 2) + 8 * a + 4 * g) = w2;
+        }
+    } else {
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+          bf16x4 wk;
+#pragma unroll
+          for (int e = 0; e < 4; e++) wk[e] = (bf16)(dk[dt][4 * a + e] * p.scale);
+          *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = wk;
+        }
+    }
   }
 }
 
-// dK, dV of a kv head = sum of the fp32 partials of its query heads; one thread per 4 elements
+// dK, dV of a kv head = sum of the fp32 partials of its query heads; one thread per 4 elements d..d+3 of the first half
+// of a key row and their partners d + 64 (the pairs of the rotary embedding)
 __global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParams p, const float* __restrict__ part) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;           // over B * Hkv * Lk * D / 4
-  const int64_t total = (int64_t)p.B * p.Hkv * p.Lk * (D / 4);
+  constexpr int Q = D / 8;                                                // threads per key row
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;           // over B * Hkv * Lk * D / 8
+  const int64_t total = (int64_t)p.B * p.Hkv * p.Lk * Q;
   if (idx >= total) return;
-  const int d4 = idx % (D / 4);
-  const int key = (idx / (D / 4)) % p.Lk;
-  const int hk = (idx / ((int64_t)(D / 4) * p.Lk)) % p.Hkv;
-  const int b = idx / ((int64_t)(D / 4) * p.Lk * p.Hkv);
+  const int d4 = idx % Q;
+  const int key = (idx / Q) % p.Lk;
+  const int hk = (idx / ((int64_t)Q * p.Lk)) % p.Hkv;
+  const int b = idx / ((int64_t)Q * p.Lk * p.Hkv);
   const int64_t plane = (int64_t)p.B * p.Hq * p.Lk * D;
-  f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = sk;
+  f32x4 sk1 = {0.f, 0.f, 0.f, 0.f}, sk2 = sk1, sv1 = sk1, sv2 = sk1;
   for (int hg = 0; hg < p.group; hg++) {
     const float* src = part + (((int64_t)b * p.Hq + hk * p.group + hg) * p.Lk + key) * D + 4 * d4;
-    sk += *reinterpret_cast<const f32x4*>(src);
-    sv += *reinterpret_cast<const f32x4*>(src + plane);
+    sk1 += *reinterpret_cast<const f32x4*>(src);
+    sk2 += *reinterpret_cast<const f32x4*>(src + D / 2);
+    sv1 += *reinterpret_cast<const f32x4*>(src + plane);
+    sv2 += *reinterpret_cast<const f32x4*>(src + plane + D / 2);
   }
-  bf16x4 wk, wv;
+  bf16x4 wk1, wk2, wv1, wv2;
+  if (p.rope_k) {
+    const bf16x8 cs = *reinterpret_cast<const bf16x8*>(p.rope_k + ((int64_t)b * p.Lk + key) * D + 8 * d4);
 #pragma unroll
-  for (int e = 0; e < 4; e++) wk[e] = (bf16)(sk[e] * p.scale), wv[e] = (bf16)sv[e];
-  *reinterpret_cast<bf16x4*>(static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l + 4 * d4) = wk;
-  *reinterpret_cast<bf16x4*>(static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l + 4 * d4) = wv;
+    for (int e = 0; e < 4; e++) {
+      const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+      const float g1 = sk1[e] * p.scale, g2 = sk2[e] * p.scale;
+      wk1[e] = (bf16)(g1 * c + g2 * sn);
+      wk2[e] = (bf16)(g2 * c - g1 * sn);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++) wk1[e] = (bf16)(sk1[e] * p.scale), wk2[e] = (bf16)(sk2[e] * p.scale);
+  }
+#pragma unroll
+  for (int e = 0; e < 4; e++) wv1[e] = (bf16)sv1[e], wv2[e] = (bf16)sv2[e];
+  bf16* dkp = static_cast<bf16*>(p.dk) + b * p.sdk.b + hk * p.sdk.h + (int64_t)key * p.sdk.l + 4 * d4;
+  bf16* dvp = static_cast<bf16*>(p.dv) + b * p.sdv.b + hk * p.sdv.h + (int64_t)key * p.sdv.l + 4 * d4;
+  *reinterpret_cast<bf16x4*>(dkp) = wk1;
+  *reinterpret_cast<bf16x4*>(dkp + D / 2) = wk2;
+  *reinterpret_cast<bf16x4*>(dvp) = wv1;
+  *reinterpret_cast<bf16x4*>(dvp + D / 2) = wv2;
 }
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
@@ -525,8 +591,8 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
     ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<true>, dim3(key_blocks * p.Hq * p.B),
                dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
     if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
-    const int64_t n4 = (int64_t)p.B * p.Hkv * p.Lk * (D / 4);
-    ODY_LAUNCH("attn_bwd_group_sum", st, attn_bwd_group_sum_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, p,
+    const int64_t n8 = (int64_t)p.B * p.Hkv * p.Lk * (D / 8);
+    ODY_LAUNCH("attn_bwd_group_sum", st, attn_bwd_group_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p,
                part);
     if ((rc = ody_check_launch("attn_bwd_group_sum"))) return rc;
   }

@@ -23,6 +23,11 @@ struct AttnParams {
   int accumulate_dq;  // bwd: dq += result
   int dq_f32;         // bwd: dq is an fp32 buffer (strides in fp32 elements) whatever the storage type of q
   int reuse_query_side;  // bwd: delta, start values and the Q / dO images in the workspace are those of the previous call
+  // bwd, bf16 head_dim 128 only: cos / sin tables (ody_rope_table layout, row pitch 128) of the query rows (B * Lq) and
+  // of the key rows (B * Lk); when set, dq and dk leave the kernels rotated back by the negative angle, i.e. as the
+  // gradient of the projection BEFORE its rotary embedding
+  const bf16* rope_q;
+  const bf16* rope_k;
   float scale;        // softmax scale
   float scale_log2e;  // scale * log2(e)
   AttnStrides sq, sk, sv, so, sdo, sdq, sdk, sdv;

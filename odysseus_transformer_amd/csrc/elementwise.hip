@@ -261,6 +261,61 @@ __global__ __launch_bounds__(256) void rope_kernel(T* __restrict__ x, const int6
   }
 }
 
+// cos / sin of every (row, frequency) once, rounded to bf16 as rope_kernel rounds them: table[row][2 j] = cos,
+// table[row][2 j + 1] = sin of pos[row] * inv_freq[j], j < D / 2.  The fused QKV projection and the attention
+// backward read it instead of evaluating sincos in their epilogues.
+__global__ __launch_bounds__(256) void rope_table_kernel(const int64_t* __restrict__ pos_ids,
+                                                         const float* __restrict__ inv_freq, int64_t rows, int D,
+                                                         float log2_base, bf16* __restrict__ table) {
+  const int half = D / 2;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * half) return;
+  const int j = idx % half;
+  const int64_t row = idx / half;
+  const float pos = pos_ids ? (float)pos_ids[row] : (float)row;
+  const float f = inv_freq ? inv_freq[j] : exp2f(-(2.0f * j / D) * log2_base);
+  const float th = pos * f;
+  typedef __attribute__((__vector_size__(2 * sizeof(bf16)))) bf16 bf16x2;
+  *reinterpret_cast<bf16x2*>(table + row * D + 2 * j) = bf16x2{(bf16)cosf(th), (bf16)sinf(th)};
+}
+
+// In-place rotation of the first n_rot heads of x (rows, heads, D) bf16 with the table above; 8 frequencies per thread.
+__global__ __launch_bounds__(256) void rope_from_table_kernel(bf16* __restrict__ x, const bf16* __restrict__ table,
+                                                              int64_t rows, int n_rot, int D, int64_t s_row, int64_t s_h,
+                                                              int inverse) {
+  const int half = D / 2, vph = half / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * vph) return;
+  const int jv = idx % vph;
+  const int64_t row = idx / vph;
+  const bf16x8 t0 = *reinterpret_cast<const bf16x8*>(table + row * D + 16 * jv);
+  const bf16x8 t1 = *reinterpret_cast<const bf16x8*>(table + row * D + 16 * jv + 8);
+  float cs[8], sn[8];
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    cs[e] = (float)t0[2 * e], sn[e] = (float)t0[2 * e + 1];
+    cs[4 + e] = (float)t1[2 * e], sn[4 + e] = (float)t1[2 * e + 1];
+  }
+  if (inverse) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) sn[e] = -sn[e];
+  }
+  bf16* base = x + row * s_row + jv * 8;
+  for (int h = 0; h < n_rot; h++) {
+    bf16* p1 = base + h * s_h;
+    bf16* p2 = p1 + half;
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(p1), c = *reinterpret_cast<const bf16x8*>(p2);
+    bf16x8 o1, o2;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      o1[e] = (bf16)((float)a[e] * cs[e] - (float)c[e] * sn[e]);
+      o2[e] = (bf16)((float)c[e] * cs[e] + (float)a[e] * sn[e]);
+    }
+    *reinterpret_cast<bf16x8*>(p1) = o1;
+    *reinterpret_cast<bf16x8*>(p2) = o2;
+  }
+}
+
 // ---------------------------------------------------------------------------
 // SwiGLU
 // ---------------------------------------------------------------------------
@@ -427,6 +482,28 @@ extern "C" int ody_rope(void* x, const int64_t* position_ids, const float* inv_f
                ODY_LAUNCH("rope", st, rope_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, (float*)x,
                                   position_ids, inv_freq, B, L, n_rot, D, sx_b, sx_l, sx_h, l2b, inverse));
   return ody_check_launch("rope");
+}
+
+extern "C" int ody_rope_table(const int64_t* position_ids, const float* inv_freq, int64_t rows, int D, float base,
+                              void* table, void* stream) {
+  ODY_REQUIRE(table, ODY_ERR_NULL, "ody_rope_table: table is NULL");
+  ODY_REQUIRE(rows > 0 && D > 0 && D % 16 == 0, ODY_ERR_BAD_SHAPE, "ody_rope_table: rows=%lld D=%d (a multiple of 16)",
+              (long long)rows, D);
+  ODY_REQUIRE(ody_aligned16(table), ODY_ERR_MISALIGNED, "ody_rope_table: table must be 16-byte aligned");
+  ODY_REQUIRE(inv_freq || base > 0.f, ODY_ERR_BAD_SHAPE, "ody_rope_table: base must be positive");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  ODY_LAUNCH("rope_table", st, rope_table_kernel, dim3(blocks_for(rows * (D / 2))), dim3(256), 0, position_ids, inv_freq,
+             rows, D, inv_freq ? 0.f : log2f(base), static_cast<bf16*>(table));
+  return ody_check_launch("rope_table");
+}
+
+// used by ody_linear_rope when the product does not take the fused kernel
+int ody_launch_rope_from_table(void* x, const void* table, int64_t rows, int n_rot, int D, int64_t s_row, int64_t s_h,
+                               int inverse, hipStream_t st) {
+  if (n_rot == 0) return ODY_OK;
+  ODY_LAUNCH("rope_from_table", st, rope_from_table_kernel, dim3(blocks_for(rows * (D / 16))), dim3(256), 0,
+             static_cast<bf16*>(x), static_cast<const bf16*>(table), rows, n_rot, D, s_row, s_h, inverse);
+  return ody_check_launch("rope_from_table");
 }
 
 namespace {

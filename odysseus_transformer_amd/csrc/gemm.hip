@@ -83,9 +83,12 @@ struct OperandTile {
 //                   even, up if odd, columns j0 + 32 (c / 2) ...), so that a lane owns gate and up of the same
 //                   (token, j).  Writes gate_up to C in its usual [gate | up] layout and h = silu(gate) * up to out2,
 //                   computed from the rounded gate / up values exactly as the stand-alone SwiGLU kernel would.
+//   EPI_ROPE        NT only, head_dim 128.  A wavefront's 128 columns are one head; columns below I (a multiple of 128)
+//                   are rotated before the one rounding: with the cos / sin table of ody_rope_table in aux (row pitch
+//                   ld_aux), column j < 64 of a head pairs with column j + 64, both in the same lane
 //   EPI_SWIGLU_BWD  the tile is dh = dy Wd (N = I); with gate_up = aux the epilogue writes d_gate_up to C (pitch
 //                   ldc, 2 I columns) as the stand-alone SwiGLU backward would from the rounded dh.
-enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU_FWD = 2, EPI_SWIGLU_BWD = 3 };
+enum { EPI_NONE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU_FWD = 2, EPI_SWIGLU_BWD = 3, EPI_ROPE = 4 };
 struct GemmEpi {
   const bf16* aux;
   bf16* out2;
@@ -105,6 +108,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
                                                              float* __restrict__ part, GemmEpi ep) {
   static_assert(EPI == EPI_NONE || (!SPLITK && WM == 4 && WN == 4), "fused epilogues: 256 x 256 tiles, one pass over K");
   static_assert(EPI != EPI_SWIGLU_FWD || (A_KC && B_KC), "the SwiGLU forward epilogue belongs to the NT product");
+  static_assert(EPI != EPI_ROPE || (A_KC && B_KC), "the rotary epilogue belongs to the NT product");
   constexpr int TM = 64 * WM, TN = 64 * WN;
   typedef OperandTile<TM, A_KC> TA;
   typedef OperandTile<TN, B_KC> TB;
@@ -188,11 +192,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
 #pragma unroll
   for (int j = 0; j < CB; j++) sstore_b(0, j);
   {
+    // in the order in which the main loop re-issues them (A and B chunks alternating): the compiler sizes the
+    // loop's s_waitcnt vmcnt for the oldest order it can see, and with all A loads ahead of all B loads here it
+    // made every B chunk's LDS store wait for loads issued half a slab ago instead of a whole one
     const int k1 = min(1, nk - 1);
+    static_assert(CA == CB, "chunks alternate");
 #pragma unroll
-    for (int j = 0; j < CA; j++) gload_a(k1, j);
-#pragma unroll
-    for (int j = 0; j < CB; j++) gload_b(k1, j);
+    for (int j = 0; j < CA; j++) {
+      gload_a(k1, j);
+      GEMM_FENCE();   // or the scheduler clusters the loads by base pointer again
+      gload_b(k1, j);
+      GEMM_FENCE();
+    }
   }
   }
   __syncthreads();
@@ -355,6 +366,46 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
         const int m = m0 + 32 * (wm * WM + a) + row;
         const int col = j0 + 32 * (wn * (WN / 2) + c / 4) + 8 * (c % 4);
         *reinterpret_cast<bf16x8*>(ep.out2 + (int64_t)m * ep.ld_out2 + col) = w;
+      }
+    }
+    return;
+  }
+  if constexpr (EPI == EPI_ROPE) {
+    constexpr int EP = 32 * WN + 8;
+    bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;
+    const bool rotate = n0 + 32 * wn * WN < ep.I;   // this wavefront's head is a query or key head
+#pragma unroll
+    for (int a = 0; a < WM; a++) {
+      const int mrow = m0 + 32 * (wm * WM + a) + i;   // the token this lane holds
+#pragma unroll
+      for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          bf16x4 w1, w2;
+          if (rotate) {
+            // (cos, sin) of frequencies 32 bb + 8 q + 4 g + (0..3): 16 bytes of the token's table row
+            const bf16x8 cs = *reinterpret_cast<const bf16x8*>(ep.aux + (int64_t)mrow * ep.ld_aux + 2 * (32 * bb + 8 * q + 4 * g));
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+              const float x1 = acc[a][bb][4 * q + e], x2 = acc[a][bb + 2][4 * q + e];
+              w1[e] = (bf16)(x1 * c - x2 * sn);
+              w2[e] = (bf16)(x2 * c + x1 * sn);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) w1[e] = (bf16)acc[a][bb][4 * q + e], w2[e] = (bf16)acc[a][bb + 2][4 * q + e];
+          }
+          *reinterpret_cast<bf16x4*>(band + i * EP + 32 * bb + 8 * q + 4 * g) = w1;
+          *reinterpret_cast<bf16x4*>(band + i * EP + 32 * (bb + 2) + 8 * q + 4 * g) = w2;
+        }
+      constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
+#pragma unroll
+      for (int pass = 0; pass < 32 / RPP; pass++) {
+        const int row = pass * RPP + lane / CPR, c = lane % CPR;
+        const bf16x8 w = *reinterpret_cast<const bf16x8*>(band + row * EP + 8 * c);
+        const int m = m0 + 32 * (wm * WM + a) + row;
+        *reinterpret_cast<bf16x8*>(C + (int64_t)m * ldc + n0 + 32 * wn * WN + 8 * c) = w;
       }
     }
     return;
@@ -944,6 +995,30 @@ int check_lin(const char* who, const void* a, const void* b, const void* c, int 
 }
 bool vec16(const void* p, int64_t ld) { return ody_aligned16(p) && ld % 8 == 0; }
 }  // namespace
+
+extern "C" int ody_linear_rope(const void* x, const void* w, const void* table, void* y, int M, int N, int K, int n_rot,
+                              int D, int64_t ldx, int64_t ldw, int64_t ld_table, int64_t ldy, int dtype, void* stream) {
+  int rc = check_lin("ody_linear_rope", x, w, y, M, N, K, dtype);
+  if (rc) return rc;
+  ODY_REQUIRE(table != nullptr, ODY_ERR_NULL, "ody_linear_rope: table is NULL");
+  ODY_REQUIRE(dtype == ODY_BF16 && D == 128, ODY_ERR_UNSUPPORTED, "ody_linear_rope: bf16 and head_dim 128 only");
+  ODY_REQUIRE(n_rot >= 0 && N % D == 0 && n_rot <= N / D, ODY_ERR_BAD_SHAPE, "ody_linear_rope: N=%d n_rot=%d D=%d", N, n_rot, D);
+  ODY_REQUIRE(ldx >= K && ldw >= K && ldy >= N, ODY_ERR_BAD_SHAPE, "ody_linear_rope: leading dimension smaller than the row length");
+  ODY_REQUIRE(ld_table == D, ODY_ERR_BAD_SHAPE, "ody_linear_rope: the table's rows are D = %d elements apart, got %lld", D,
+              (long long)ld_table);
+  ODY_REQUIRE(vec16(table, ld_table) && vec16(y, ldy), ODY_ERR_MISALIGNED,
+              "ody_linear_rope: table and y need 16-byte aligned rows");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (fused_shape_ok(M, N, K, ldx, ldw) && vec16(x, ldx) && vec16(w, ldw)) {
+    GemmEpi ep{static_cast<const bf16*>(table), nullptr, ld_table, 0, n_rot * D};
+    return launch_fused<true, EPI_ROPE>("gemm_bf16_nt_rope", static_cast<const bf16*>(x), static_cast<const bf16*>(w),
+                                        static_cast<bf16*>(y), M, N, K, ldx, ldw, ldy, ep, st);
+  }
+  // other shapes: the plain product, then the rotation in place (one more rounding of the rotated columns)
+  rc = ody_gemm(ODY_GEMM_NT, x, w, y, nullptr, M, N, K, ldx, ldw, ldy, 0, dtype, nullptr, 0, stream);
+  if (rc) return rc;
+  return ody_launch_rope_from_table(y, table, M, n_rot, D, ldy, D, 0, st);
+}
 
 extern "C" int ody_linear_residual(const void* x, const void* w, const void* residual, void* y, int M, int N, int K,
                                    int64_t ldx, int64_t ldw, int64_t ld_res, int64_t ldy, int dtype, void* stream) {

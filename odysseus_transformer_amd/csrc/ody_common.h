@@ -27,6 +27,10 @@ int ody_check_launch(const char* what);
 // Raises a kernel's dynamic-LDS limit to `bytes` on the current device.  Done once per (kernel, device)
 // under a lock, so concurrent first calls from several host threads and several devices are safe.
 int ody_allow_dynamic_lds(const void* kernel, size_t bytes, const char* who);
+// In-place rotation (inverse != 0: by the negative angle) of the first n_rot heads of a bf16 (rows, heads, D) array with
+// the cos / sin table of ody_rope_table; s_row, s_h in elements.
+int ody_launch_rope_from_table(void* x, const void* table, int64_t rows, int n_rot, int D, int64_t s_row, int64_t s_h,
+                               int inverse, hipStream_t st);
 
 // Brackets one kernel launch with a pair of HIP events on the launch stream when the
 // timer is enabled (ody_profile_enable); costs one branch otherwise.

@@ -104,6 +104,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
         self.max_position_embeddings = getattr(config, "max_position_embeddings", None)
         self.rope_theta = _rope_theta(config)
         self.is_causal = True
+        self.fuse_rope = True   # rotary embedding inside the QKV projection and the attention backward when possible
 
         self.model_parallel_size = get_model_parallel_world_size()
         self.local_rank = get_model_parallel_rank()
@@ -151,8 +152,14 @@ class LlamaFlashAttention2TPSP(nn.Module):
             q_len = local_q_len * get_model_parallel_world_size()
             if not self.sequence_parallel:
                 hidden_states = allgather_bsz1(hidden_states)
-            qkv3, attn_output, _ = PackedRoPEAttnFunc.apply(self.qkv_proj(hidden_states), nh, nkv, D, position_ids,
-                                                            self.rope_theta, scale)
+            if self._can_fuse_rope(hidden_states):
+                # projection, rotary embedding and attention as one autograd node: the rotation rides in the
+                # projection's epilogue, its backward in the epilogues of the attention backward
+                qkv3, attn_output, _ = ops.QKVRoPEAttnFunc.apply(hidden_states, self.qkv_proj.weight, nh, nkv, D,
+                                                                 position_ids, self.rope_theta, scale)
+            else:
+                qkv3, attn_output, _ = PackedRoPEAttnFunc.apply(self.qkv_proj(hidden_states), nh, nkv, D, position_ids,
+                                                                self.rope_theta, scale)
             if past_key_value is not None:
                 qkv = qkv3.detach().view(bsz, q_len, nh + 2 * nkv, D)
                 self._update_cache(past_key_value, qkv[:, :, nh:nh + nkv], qkv[:, :, nh + nkv:], q_len, cache_position)
@@ -180,6 +187,15 @@ class LlamaFlashAttention2TPSP(nn.Module):
         if self.return_arity == 2:
             return attn_output, None
         return attn_output, None, past_key_value
+
+    def _can_fuse_rope(self, hidden_states) -> bool:
+        """The fused node stands for gather(x) W^T followed by the rotation, which is what the packed projection
+        computes when the gather is the identity (one rank), there is no bias and autocast asks for no cast;
+        the fused kernels exist for bfloat16 and head_dim 128."""
+        return (self.fuse_rope and self.head_dim == 128 and get_model_parallel_world_size() == 1
+                and self.qkv_proj.bias is None and hidden_states.dtype == torch.bfloat16
+                and self.qkv_proj.weight.dtype == torch.bfloat16 and hidden_states.is_cuda
+                and not torch.is_autocast_enabled("cuda"))
 
     def _can_fuse_residual(self, residual, attn_output) -> bool:
         """The epilogue add stands for reduce_scatter(x W^T) + residual, which is only the same thing when the
@@ -263,6 +279,7 @@ class OdysseusDecoderLayer(nn.Module):
         self.self_attn = LlamaFlashAttention2TPSP(config, layer_idx)
         self.mlp = LlamaMLPZeRO(config)
         self.mlp.fuse_elementwise = fused
+        self.self_attn.fuse_rope = fused
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
 

@@ -110,13 +110,15 @@ def attn_fwd_noalloc(q, k, v, out, lse, causal: bool = True, scale: Optional[flo
 
 
 def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
-             dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False):
+             dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False,
+             rope_tables=None):
     """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.
 
     dq may be a float32 tensor although q is bfloat16: with accumulate_dq that is the running dq of a
     ring step, summed exactly over the key blocks.  reuse_query_side=True (needs the `workspace` of
     the previous call, with the same q / out / lse / dout) skips the scratch that depends on the
-    queries only."""
+    queries only.  rope_tables=(table_q, table_k) (rope_table() of the query / key positions; bf16,
+    head_dim 128) makes dq and dk the gradients of the projection BEFORE its rotary embedding."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
@@ -148,11 +150,20 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
             (_lib.BWD_REUSE_QUERY_SIDE if reuse_query_side else 0)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
-    _lib.call("ody_attn_bwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-              dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-              B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
-              *_blhd(dout, "dout"), *_blhd(dq, "dq"), *_blhd(dk, "dk"), *_blhd(dv, "dv"),
-              scale, int(causal), flags, _dt(q), ws.data_ptr(), ws_bytes, _stream())
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
+            *_blhd(dout, "dout"), *_blhd(dq, "dq"), *_blhd(dk, "dk"), *_blhd(dv, "dv"),
+            scale, int(causal), flags, _dt(q), ws.data_ptr(), ws_bytes, _stream())
+    if rope_tables is None:
+        _lib.call("ody_attn_bwd", *args)
+    else:
+        tq, tk = rope_tables
+        for t, n, rows in ((tq, "table_q", B * Lq), (tk, "table_k", B * Lk)):
+            _need_gpu(t)
+            if t.dtype != torch.bfloat16 or not t.is_contiguous() or tuple(t.shape) != (rows, D) or t.device != q.device:
+                raise ValueError(f"{n} must be a contiguous bfloat16 ({rows}, {D}) tensor on {q.device}")
+        _lib.call("ody_attn_bwd_rope", *args, tq.data_ptr(), tk.data_ptr())
     return dq, dk, dv
 
 
@@ -248,6 +259,62 @@ def linear_residual(x, weight, residual):
     _lib.call("ody_linear_residual", x.data_ptr(), weight.data_ptr(), residual.data_ptr(), y.data_ptr(), M, N, K,
               _rowmajor2d(x, "x"), _rowmajor2d(weight, "weight"), _rowmajor2d(residual, "residual"), y.stride(0),
               _dt(x), _stream())
+    return y
+
+
+_ROPE_TABLE_LAST = None   # (position tensor, its version, rows, head_dim, base, device, stream, table) of the last table built
+
+
+def rope_table(position_ids, rows: int, head_dim: int, base: float = 10000.0, device=None, inv_freq=None) -> torch.Tensor:
+    """(rows, head_dim) bfloat16: [r, 2 j] = cos, [r, 2 j + 1] = sin of position r times frequency j, rounded
+    as rope_ rounds them.  position_ids: int64 with `rows` elements in the order of the rows, or None for arange.
+
+    The layers of a model are handed one and the same position tensor: the last table is kept and returned again
+    for the same tensor object (unmodified since), shape, base and stream.  Treat the result as read-only."""
+    global _ROPE_TABLE_LAST
+    pos_arg = position_ids
+    if position_ids is not None:
+        _need_gpu(position_ids)
+        device = position_ids.device
+    if device is None:
+        raise ValueError("rope_table needs position_ids or a device")
+    device = torch.device(device)
+    key = (None if pos_arg is None else pos_arg._version, rows, head_dim, float(base), str(device), _stream())
+    last = _ROPE_TABLE_LAST
+    if inv_freq is None and last is not None and last[0] is pos_arg and last[1] == key:
+        return last[2]
+    if position_ids is not None:
+        position_ids = position_ids.to(torch.int64).reshape(-1).contiguous()
+        if position_ids.numel() != rows:
+            raise ValueError(f"{position_ids.numel()} positions for {rows} rows")
+    custom_freq = inv_freq is not None
+    if inv_freq is None:
+        inv_freq = rope_inv_freq(head_dim, base, device)
+    if inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2 or not inv_freq.is_contiguous():
+        raise ValueError("inv_freq must be a contiguous float32 tensor of head_dim / 2 elements")
+    table = torch.empty((rows, head_dim), dtype=torch.bfloat16, device=device)
+    _lib.call("ody_rope_table", position_ids.data_ptr() if position_ids is not None else 0, inv_freq.data_ptr(), rows,
+              head_dim, float(base), table.data_ptr(), _stream())
+    if not custom_freq:
+        _ROPE_TABLE_LAST = (pos_arg, key, table)   # holding pos_arg keeps its identity from being reused
+    return table
+
+
+def linear_rope(x, weight, table, n_rot: int, head_dim: int):
+    """x (M, K) W (N, K)^T with the first n_rot heads of head_dim columns rotated by row m of `table`
+    (rope_table) in the product's epilogue: the packed QKV projection and its rotary embedding in one kernel."""
+    _need_gpu(x, weight, table)
+    _lin_args(x, weight, "linear_rope")
+    (M, K), N = x.shape, weight.shape[0]
+    if weight.shape[1] != K or N % head_dim or not 0 <= n_rot <= N // head_dim:
+        raise ValueError(f"linear_rope: x {tuple(x.shape)}, weight {tuple(weight.shape)}, n_rot {n_rot}, head_dim {head_dim}")
+    if x.dtype != torch.bfloat16 or head_dim != 128:
+        raise ValueError("linear_rope: bfloat16 and head_dim 128 only")
+    if table.dtype != torch.bfloat16 or tuple(table.shape) != (M, head_dim) or not table.is_contiguous():
+        raise ValueError(f"linear_rope: table must be a contiguous bfloat16 ({M}, {head_dim}) tensor")
+    y = torch.empty((M, N), dtype=x.dtype, device=x.device)
+    _lib.call("ody_linear_rope", x.data_ptr(), weight.data_ptr(), table.data_ptr(), y.data_ptr(), M, N, K, n_rot, head_dim,
+              _rowmajor2d(x, "x"), _rowmajor2d(weight, "weight"), table.stride(0), y.stride(0), _dt(x), _stream())
     return y
 
 
@@ -658,6 +725,46 @@ class LinearResidualFunc(torch.autograd.Function):
         x2 = x.reshape(-1, x.shape[-1])
         dw = gemm(GEMM_TN, dy2, x2 if x2.stride(1) == 1 else x2.contiguous())
         return dx, dw, dy
+
+
+class QKVRoPEAttnFunc(torch.autograd.Function):
+    """Packed QKV projection, rotary embedding of q and k and causal GQA attention with no separate rotary
+    pass (bf16, head_dim 128): forward rotates in the projection's epilogue, backward un-rotates dq and dk in the
+    epilogues of the attention backward (decoder/odysseus.py:180-263 of the reference, utils/linear_tpsp.py:173,
+    217,291 for the three products).  Returns (qkv, out, lse); qkv is the rotated projection (for a KV cache)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, n_heads, n_kv_heads, head_dim, position_ids, rope_base, softmax_scale):
+        B, L, K = x.shape
+        x2 = x.reshape(B * L, K)
+        x2 = x2 if x2.stride(1) == 1 else x2.contiguous()
+        pos = position_ids
+        if pos is not None and pos.numel() != B * L:
+            pos = pos.expand(B, L)
+        table = rope_table(pos, B * L, head_dim, rope_base, device=x.device)
+        H = n_heads + 2 * n_kv_heads
+        qkv = linear_rope(x2, weight, table, n_heads + n_kv_heads, head_dim).view(B, L, H, head_dim)
+        a, b = n_heads, n_heads + n_kv_heads
+        out, lse = attn_fwd(qkv[:, :, :a], qkv[:, :, a:b], qkv[:, :, b:], causal=True, scale=softmax_scale)
+        ctx.save_for_backward(x2, weight, qkv, out, lse, table)
+        ctx.dims = (n_heads, n_kv_heads, head_dim, softmax_scale, x.shape)
+        ctx.mark_non_differentiable(lse, qkv)
+        return qkv, out, lse
+
+    @staticmethod
+    def backward(ctx, _dqkv, dout, _dlse):
+        x2, weight, qkv, out, lse, table = ctx.saved_tensors
+        n_heads, n_kv_heads, head_dim, softmax_scale, x_shape = ctx.dims
+        if dout.stride(3) != 1:
+            dout = dout.contiguous()
+        dqkv = torch.empty_like(qkv)
+        a, b = n_heads, n_heads + n_kv_heads
+        attn_bwd(qkv[:, :, :a], qkv[:, :, a:b], qkv[:, :, b:], out, lse, dout, causal=True, scale=softmax_scale,
+                 dq=dqkv[:, :, :a], dk=dqkv[:, :, a:b], dv=dqkv[:, :, b:], rope_tables=(table, table))
+        d2 = dqkv.view(x2.shape[0], -1)
+        dx = gemm(GEMM_NN, d2, weight).view(x_shape)
+        dw = gemm(GEMM_TN, d2, x2)
+        return dx, dw, None, None, None, None, None, None
 
 
 class SwiGLUMLPResidualFunc(torch.autograd.Function):

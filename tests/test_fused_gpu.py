@@ -126,3 +126,121 @@ def test_fused_layer_matches_the_unfused_layer_and_the_oracle(L, d, H, Hkv, D, i
     assert_parity(dxf, g_ref["x"], tol, "dx")
     for k, v in p.items():
         assert rel_err(v.grad, g_ref[k]) <= tol, k
+
+
+# ----------------------------------------------------------------------------------------------
+# rotary embedding inside the QKV projection and the attention backward
+# ----------------------------------------------------------------------------------------------
+def _rope_ref(x4, pos, base=10000.0):
+    """fp32 rotation of (B, L, H, D) by the oracle's cos / sin."""
+    cos, sin = oracle.rope_cos_sin(pos, x4.shape[-1], base, torch.float32)
+    return oracle.apply_rope(x4.float(), cos, sin)
+
+
+def test_rope_table_holds_the_rounded_cos_and_sin(dev):
+    from odysseus_transformer_amd import ops
+    pos = torch.tensor([[0, 1, 5, 1000, 65535, 1048575]])
+    t = ops.rope_table(pos.to(dev), 6, 128, 10000.0).float().cpu()
+    cos, sin = oracle.rope_cos_sin(pos, 128, 10000.0, torch.float32)       # (1, 6, 128): [freqs, freqs]
+    assert (t[:, 0::2] - cos[0, :, :64]).abs().max() <= 2 ** -8            # bf16 rounding of values in [-1, 1]
+    assert (t[:, 1::2] - sin[0, :, :64]).abs().max() <= 2 ** -8
+    t2 = ops.rope_table(None, 4, 128, 10000.0, device=dev).float().cpu()   # no positions: the row index
+    cos, sin = oracle.rope_cos_sin(torch.arange(4)[None], 128, 10000.0, torch.float32)
+    assert (t2[:, 0::2] - cos[0, :, :64]).abs().max() <= 2 ** -8
+
+
+@pytest.mark.parametrize("M,N,K,n_rot", [(512, 768, 256, 4), (256, 1536, 4096, 8), (300, 384, 200, 2), (512, 512, 320, 0)])
+def test_linear_rope_against_the_product_followed_by_the_rotation(M, N, K, n_rot, dev):
+    """Fused kernel (whole 256 x 256 tiles, K a multiple of 64) and the two-kernel path for other shapes."""
+    from odysseus_transformer_amd import ops
+    x = randn((M, K), 9300, dtype=torch.bfloat16)
+    w = randn((N, K), 9301, std=0.05, dtype=torch.bfloat16)
+    pos = torch.randint(0, 40000, (1, M), generator=torch.Generator().manual_seed(9302))
+    table = ops.rope_table(pos.to(dev), M, 128, 10000.0)
+    y = ops.linear_rope(x.to(dev), w.to(dev), table, n_rot, 128)
+    y_ref = oracle.linear_fwd(x.float(), w.float()).view(1, M, N // 128, 128)
+    y_ref = torch.cat((_rope_ref(y_ref[:, :, :n_rot], pos), y_ref[:, :, n_rot:]), dim=2).reshape(M, N)
+    assert_parity(y, y_ref, 1e-2, "rotated projection")     # bf16 cos / sin and one (fused) or two roundings
+
+
+@pytest.mark.parametrize("L,Hq,Hkv,B", [(512, 4, 4, 1), (300, 4, 1, 1), (260, 2, 2, 2), (1024, 8, 2, 1)])
+def test_attention_backward_with_the_inverse_rotation_in_its_epilogues(L, Hq, Hkv, B, dev):
+    """dq and dk of ody_attn_bwd_rope against ody_attn_bwd followed by the inverse rotation: the one-kernel-per-key-head
+    and the per-query-head (group sum) variants of the dK / dV kernel, ragged lengths, two batches."""
+    from odysseus_transformer_amd import ops
+    D = 128
+    q, k, v, do = (randn((B, L, h, D), 9400 + n, dtype=torch.bfloat16).to(dev) for n, h in enumerate((Hq, Hkv, Hkv, Hq)))
+    pos = torch.randint(0, 100000, (B, L), generator=torch.Generator().manual_seed(9404)).to(dev)
+    out, lse = ops.attn_fwd(q, k, v, causal=True)
+    dq0, dk0, dv0 = ops.attn_bwd(q, k, v, out, lse, do, causal=True)
+    ops.rope_(dq0, Hq, pos, 10000.0, inverse=True)
+    ops.rope_(dk0, Hkv, pos, 10000.0, inverse=True)
+    table = ops.rope_table(pos, B * L, D, 10000.0)
+    dq1, dk1, dv1 = ops.attn_bwd(q, k, v, out, lse, do, causal=True, rope_tables=(table, table))
+    torch.cuda.synchronize()
+    assert torch.equal(dv1, dv0)
+    assert_parity(dq1, dq0.float(), 8e-3, "dq", seq_dim=1)     # the fused path rounds once, the other twice
+    assert_parity(dk1, dk0.float(), 8e-3, "dk", seq_dim=1)
+    with pytest.raises(Exception):
+        ops.attn_bwd(q, k, v, out, lse, do, causal=True, dq=dq1, accumulate_dq=True, rope_tables=(table, table))
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (4, 2)])
+def test_attention_module_with_and_without_the_fused_rotation(Hq, Hkv, dev):
+    """LlamaFlashAttention2TPSP forward and every gradient: fused node (projection + rotation + attention) against the
+    chain of separate kernels and against the oracle."""
+    import types
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    L, d, D = 512, 512, 128
+    cfg = types.SimpleNamespace(hidden_size=d, num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D,
+                                intermediate_size=1024, hidden_act="silu", attention_dropout=0.0, rms_norm_eps=1e-6,
+                                rope_theta=10000.0, max_position_embeddings=1 << 20, pretraining_tp=1, num_hidden_layers=1)
+    x = randn((1, L, d), 9500, dtype=torch.bfloat16)
+    dy = randn((1, L, d), 9501, dtype=torch.bfloat16)
+    w_qkv = randn(((Hq + 2 * Hkv) * D, d), 9502, std=0.05, dtype=torch.bfloat16)
+    w_o = randn((d, Hq * D), 9503, std=0.05, dtype=torch.bfloat16)
+    res = {}
+    for fused in (True, False):
+        attn = LlamaFlashAttention2TPSP(cfg, 0).to(torch.bfloat16).to(dev)
+        attn.fuse_rope = fused
+        with torch.no_grad():
+            attn.qkv_proj.weight.copy_(w_qkv)
+            attn.o_proj.weight.copy_(w_o)
+        xg = x.to(dev).requires_grad_(True)
+
+        def step():
+            y = attn(xg, position_ids=torch.arange(L, device=dev)[None])[0]
+            y.backward(dy.to(dev))
+            return y
+        y, names = _kernels_of(step)
+        assert ("rope" in names) == (not fused), names
+        assert ("gemm_bf16_nt_rope" in names) == fused, names
+        res[fused] = [t.float().cpu() for t in (y, xg.grad, attn.qkv_proj.weight.grad, attn.o_proj.weight.grad)]
+    # oracle: projection -> rotation -> attention -> projection, explicit backward
+    pos = torch.arange(L)[None]
+    qkv = oracle.linear_fwd(x.float(), w_qkv.float())
+    q0, k0, v0 = oracle.split_qkv(qkv, Hq, Hkv, D)
+    cos, sin = oracle.rope_cos_sin(pos, D, 10000.0, torch.float32)
+    q, k = oracle.apply_rope(q0, cos, sin), oracle.apply_rope(k0, cos, sin)
+    o, lse = oracle.attention_fwd(q, k, v0, causal=True)
+    y_ref = oracle.linear_fwd(o.reshape(1, L, Hq * D), w_o.float())
+    do2, dwo_ref, _ = oracle.linear_bwd(o.reshape(1, L, Hq * D), w_o.float(), dy.float())
+    dq, dk, dv = oracle.attention_bwd(q, k, v0, o, lse, do2.view(1, L, Hq, D), causal=True)
+    dqkv = torch.cat((oracle.apply_rope_bwd(dq, cos, sin), oracle.apply_rope_bwd(dk, cos, sin), dv), dim=2)
+    dx_ref, dwqkv_ref, _ = oracle.linear_bwd(x.float(), w_qkv.float(), dqkv.reshape(1, L, -1))
+    for fused in (True, False):
+        for got, ref, what in zip(res[fused], (y_ref, dx_ref, dwqkv_ref, dwo_ref), ("y", "dx", "dWqkv", "dWo")):
+            assert_parity(got, ref, TOL_BF16, f"fused={fused} {what}")
+
+
+def test_rope_table_is_reused_for_the_same_position_tensor_only(dev):
+    from odysseus_transformer_amd import ops
+    pos = torch.arange(64, device=dev)[None]
+    t1 = ops.rope_table(pos, 64, 128, 10000.0)
+    assert ops.rope_table(pos, 64, 128, 10000.0) is t1                 # the next layer of the same forward pass
+    assert ops.rope_table(pos, 64, 128, 500000.0) is not t1            # another base
+    t3 = ops.rope_table(pos.clone(), 64, 128, 10000.0)                 # another tensor object
+    assert t3 is not t1 and torch.equal(t3, t1)
+    pos.add_(7)                                                        # modified in place: built again
+    t4 = ops.rope_table(pos, 64, 128, 10000.0)
+    assert ops.rope_table(pos, 64, 128, 10000.0) is t4 and not torch.equal(t4, t3)

@@ -28,13 +28,14 @@ def _oracle_attention_block_fwd_bwd(x, w_qkv, w_o, dy, H, Hkv, D, note, storage=
     """The oracle's functions composed as decoder/odysseus.py:170-271 orders them, with the explicit
     backward: returns y and the gradients of x, w_qkv, w_o.  With `storage` set, every tensor that
     the bf16 pipeline (the reference's as much as this one) keeps in memory between two operations
-    -- projection output, rotary table, rotated q / k, attention output, and their gradients -- is
-    rounded to that type; the arithmetic stays fp32."""
+    -- rotary table, rotated q / k, v, attention output, and their gradients -- is rounded to that
+    type; the arithmetic stays fp32."""
     r = (lambda t: t) if storage is None else (lambda t: t.to(storage).float())
     B, L, _ = x.shape
     pos = torch.arange(L)[None]
-    qkv = r(oracle.linear_fwd(x, w_qkv))
-    q0, k0, v = oracle.split_qkv(qkv, H, Hkv, D)
+    # the rotation rides in the projection's epilogue: q and k are rounded once, after it; v as it leaves the product
+    q0, k0, v = oracle.split_qkv(oracle.linear_fwd(x, w_qkv), H, Hkv, D)
+    v = r(v)
     cos, sin = oracle.rope_cos_sin(pos, D, 10000.0, x.dtype)
     cos, sin = r(cos), r(sin)
     q, k = r(oracle.apply_rope(q0, cos, sin)), r(oracle.apply_rope(k0, cos, sin))
@@ -46,7 +47,8 @@ def _oracle_attention_block_fwd_bwd(x, w_qkv, w_o, dy, H, Hkv, D, note, storage=
     do2, dw_o, _ = oracle.linear_bwd(o2, w_o, dy)
     dq, dk, dv = oracle.attention_bwd(q, k, v, o, lse, r(do2).view(B, L, H, D), causal=True)
     print(f"  {note}: oracle attention backward done", flush=True)
-    dqkv = r(torch.cat((oracle.apply_rope_bwd(r(dq), cos, sin), oracle.apply_rope_bwd(r(dk), cos, sin), dv), dim=2))
+    # likewise dq and dk are rotated back in the attention backward's epilogues, before their one rounding
+    dqkv = r(torch.cat((oracle.apply_rope_bwd(dq, cos, sin), oracle.apply_rope_bwd(dk, cos, sin), dv), dim=2))
     dx, dw_qkv, _ = oracle.linear_bwd(x, w_qkv, dqkv.reshape(B, L, -1))
     return y, dx, dw_qkv, dw_o
 
