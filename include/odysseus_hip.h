@@ -308,6 +308,17 @@ int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o
                       void* workspace, size_t workspace_bytes, void* stream,
                       const void* rope_table_q, const void* rope_table_k);
 
+/* ---- optimizer ------------------------------------------------------------
+ * One step of torch.optim.AdamW (the optimizer of the reference's training loop, train.py:170,216) on one
+ * tensor of n elements, in one pass instead of the host framework's seven element-wise passes:
+ *   p *= 1 - lr * weight_decay;  m = beta1 m + (1 - beta1) g;  v = beta2 v + (1 - beta2) g^2;
+ *   p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps)
+ * param, grad, exp_avg, exp_avg_sq: contiguous arrays of `dtype`, 16-byte aligned; fp32 arithmetic, one rounding per
+ * stored value.  step counts from 1.
+ */
+int ody_adamw(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, int64_t n, float lr, float beta1,
+              float beta2, float eps, float weight_decay, int64_t step, int dtype, void* stream);
+
 /* ---- cross-entropy over the vocabulary --------------------------------------
  * flash_attn.losses.cross_entropy.CrossEntropyLoss(inplace_backward=True) as the training loop
  * uses it (train.py:8,173,212-214): softmax cross-entropy of logits (T, V) (row stride ld,

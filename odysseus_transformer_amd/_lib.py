@@ -49,6 +49,7 @@ SIGNATURES = {
     "ody_cross_entropy_bwd": (_i, [_p] * 6 + [_i, _i, _i64, _i64, _i, _p]),
     "ody_rope": (_i, [_p, _p, _p, _i, _i, _i, _i, _i64, _i64, _i64, _f, _i, _i, _p]),
     "ody_rope_table": (_i, [_p, _p, _i64, _i, _f, _p, _p]),
+    "ody_adamw": (_i, [_p, _p, _p, _p, _i64, _f, _f, _f, _f, _f, _i64, _i, _p]),
     "ody_linear_rope": (_i, [_p] * 4 + [_i] * 5 + [_i64] * 4 + [_i, _p]),
     "ody_attn_bwd_rope": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p, _p, _p]),
 }

@@ -2,6 +2,8 @@
 // All move 16-byte vectors per lane, keep statistics in fp32 and reduce inside a
 // wavefront with lane shuffles; none of them is shaped into a matrix product.
 #include <cmath>
+#include <algorithm>
+#include <cmath>
 #include "ody_common.h"
 
 namespace {
@@ -592,4 +594,69 @@ extern "C" int ody_lse_merge(float* out_acc, float* lse_acc, const void* out_blk
                ODY_LAUNCH("lse_merge", st, lse_merge_kernel<float>, dim3(blocks_for(total)), dim3(256), 0, out_acc, lse_acc,
                                   (const float*)out_blk, lse_blk, B, L, H, D, sb_b, sb_l, sb_h));
   return ody_check_launch("lse_merge");
+}
+
+// ---------------------------------------------------------------------------
+// AdamW, one pass: torch.optim.AdamW's update (train.py:170,216 of the reference) on one tensor.  Memory-bound:
+// parameter, gradient and both moments are read once, parameter and moments written once (14 bytes per bf16
+// parameter); the arithmetic is fp32 whatever the storage type, with one rounding per stored value.
+//   p *= 1 - lr * wd;  m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g^2;  p -= (lr / bc1) * m / (sqrt(v) / sqrt(bc2) + eps)
+// ---------------------------------------------------------------------------
+namespace {
+template <typename T>
+__global__ __launch_bounds__(256) void adamw_kernel(T* __restrict__ p, const T* __restrict__ g, T* __restrict__ m,
+                                                    T* __restrict__ v, int64_t n, float decay, float b1, float b2,
+                                                    float step_size, float inv_sqrt_bc2, float eps) {
+  constexpr int N = VecIO<T>::N;
+  const int64_t nv = n / N;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += (int64_t)gridDim.x * 256) {
+    float pf[N], gf[N], mf[N], vf[N];
+    VecIO<T>::load(p + i * N, pf);
+    VecIO<T>::load(g + i * N, gf);
+    VecIO<T>::load(m + i * N, mf);
+    VecIO<T>::load(v + i * N, vf);
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      mf[e] = b1 * mf[e] + (1.f - b1) * gf[e];
+      vf[e] = b2 * vf[e] + (1.f - b2) * gf[e] * gf[e];
+      pf[e] = pf[e] * decay - step_size * mf[e] / (sqrtf(vf[e]) * inv_sqrt_bc2 + eps);
+    }
+    VecIO<T>::store(p + i * N, pf);
+    VecIO<T>::store(m + i * N, mf);
+    VecIO<T>::store(v + i * N, vf);
+  }
+  // the tail that does not fill a 16-byte vector
+  if (blockIdx.x == 0 && threadIdx.x < n - nv * N) {
+    const int64_t i = nv * N + threadIdx.x;
+    const float gf = (float)g[i];
+    const float mf = b1 * (float)m[i] + (1.f - b1) * gf;
+    const float vf = b2 * (float)v[i] + (1.f - b2) * gf * gf;
+    p[i] = (T)((float)p[i] * decay - step_size * mf / (sqrtf(vf) * inv_sqrt_bc2 + eps));
+    m[i] = (T)mf;
+    v[i] = (T)vf;
+  }
+}
+}  // namespace
+
+extern "C" int ody_adamw(void* param, const void* grad, void* exp_avg, void* exp_avg_sq, int64_t n, float lr, float beta1,
+                         float beta2, float eps, float weight_decay, int64_t step, int dtype, void* stream) {
+  ODY_REQUIRE(param && grad && exp_avg && exp_avg_sq, ODY_ERR_NULL, "ody_adamw: NULL pointer");
+  ODY_REQUIRE(n > 0 && step >= 1, ODY_ERR_BAD_SHAPE, "ody_adamw: n=%lld step=%lld", (long long)n, (long long)step);
+  ODY_REQUIRE(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f && eps >= 0.f, ODY_ERR_BAD_SHAPE,
+              "ody_adamw: betas (%g, %g) in [0, 1), eps %g >= 0", beta1, beta2, eps);
+  ODY_REQUIRE(ody_aligned16(param) && ody_aligned16(grad) && ody_aligned16(exp_avg) && ody_aligned16(exp_avg_sq),
+              ODY_ERR_MISALIGNED, "ody_adamw: pointers must be 16-byte aligned");
+  const double bc1 = 1.0 - pow((double)beta1, (double)step), bc2 = 1.0 - pow((double)beta2, (double)step);
+  const float step_size = (float)((double)lr / bc1), inv_sqrt_bc2 = (float)(1.0 / sqrt(bc2));
+  const float decay = 1.f - lr * weight_decay;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int per = dtype == ODY_BF16 ? 8 : 4;
+  const int64_t nv = n / per;
+  const unsigned blocks = (unsigned)std::min<int64_t>(std::max<int64_t>((nv + 255) / 256, 1), 256 * 16);
+  ODY_BY_DTYPE(dtype,
+               ODY_LAUNCH("adamw", st, adamw_kernel<bf16>, dim3(blocks), dim3(256), 0, (bf16*)param, (const bf16*)grad,
+                          (bf16*)exp_avg, (bf16*)exp_avg_sq, n, decay, beta1, beta2, step_size, inv_sqrt_bc2, eps),
+               ODY_LAUNCH("adamw", st, adamw_kernel<float>, dim3(blocks), dim3(256), 0, (float*)param, (const float*)grad,
+                          (float*)exp_avg, (float*)exp_avg_sq, n, decay, beta1, beta2, step_size, inv_sqrt_bc2, eps));
+  return ody_check_launch("adamw");
 }

@@ -17,7 +17,9 @@ branch skips it too, train.py:118); `--native-host-modules` (default on) also ro
 model's RMSNorms, lm_head and whatever bias-free projections the patch left in its layers through
 the HIP library, so that the step runs on this library's kernels except for the embedding lookup,
 the residual adds (and, in the ulysses / ring / dp modes, the rotary embedding and SiLU-multiply)
-of the host decoder layer and the optimizer; switch it off to keep every host module as transformers ships it.
+of the host decoder layer; `--native-optimizer` (default on) runs AdamW as one kernel per tensor
+(odysseus_transformer_amd.optim.AdamW) instead of the host framework's element-wise passes.  Switch
+either off to keep the host's own modules / optimizer.
 """
 from __future__ import annotations
 
@@ -139,7 +141,11 @@ def main(args) -> dict:
     mem = lambda: (torch.cuda.memory_allocated(dev) / 1024 ** 3, torch.cuda.memory_reserved(dev) / 1024 ** 3)
     print(f"{args.parallel_mode} After init model, CUDA memory allocated: {mem()[0]:.2f} GB, reserved: {mem()[1]:.2f} GB")
 
-    optim = torch.optim.AdamW(model.parameters(), lr=args.learning_rate)
+    if args.native_optimizer:
+        from .optim import AdamW                      # the same update in one pass per tensor
+        optim = AdamW(model.parameters(), lr=args.learning_rate)
+    else:
+        optim = torch.optim.AdamW(model.parameters(), lr=args.learning_rate)
     model.train()
     loss_func = CrossEntropyLoss(inplace_backward=True)
     warmup_num_iterations = 2
@@ -163,8 +169,11 @@ def main(args) -> dict:
         loss.backward(loss)
         optim.step()
         optim.zero_grad()
+        if step >= warmup_num_iterations:
+            # the reference starts and stops its clock without one, so that a timed step pays for the queued tail of the
+            # step before it; here the seven timed steps are seven whole steps
+            torch.cuda.synchronize()
         if step > warmup_num_iterations:
-            torch.cuda.synchronize()                  # the reference stops its clock without one; the next loss.item() pays for it there
             step_times.append(time.time() - start_time)
             elapse += step_times[-1]
     print(f"{args.parallel_mode} {args.seq_length//1024}K {world_size} Time taken: {elapse:.2f} seconds")
@@ -173,7 +182,7 @@ def main(args) -> dict:
            "step_ms": [round(1e3 * t, 1) for t in step_times], "tokens_per_s": round(args.seq_length * len(step_times) /
                                                                                       max(elapse, 1e-9), 1),
            "peak_memory_gb": round(torch.cuda.max_memory_allocated(dev) / 1024 ** 3, 2), "losses": [round(l, 4) for l in losses],
-           "native_host_modules": bool(args.native_host_modules)}
+           "native_host_modules": bool(args.native_host_modules), "native_optimizer": bool(args.native_optimizer)}
     print(json.dumps(out))
     return out
 
@@ -192,6 +201,8 @@ def parse_args(argv=None):
     ap.add_argument("--parallel_mode", type=str, choices=["odysseus", "ulysses", "dp", "tpsp", "ring"], default="odysseus")
     ap.add_argument("--num-hidden-layers", type=int, default=16, help="16 in the reference's configuration (train.py:71)")
     ap.add_argument("--native-host-modules", action=argparse.BooleanOptionalAction, default=True)
+    ap.add_argument("--native-optimizer", action=argparse.BooleanOptionalAction, default=True,
+                    help="AdamW as one HIP kernel per tensor instead of torch.optim.AdamW's element-wise passes")
     ap.add_argument("--declare-flash-attention", action=argparse.BooleanOptionalAction, default=False,
                     help="set config._attn_implementation before the model is built (needs flash_attn importable); "
                          "the patchers set it afterwards either way")

@@ -33,6 +33,8 @@ How each function is pinned (tests/test_oracle.py):
                      formula with gate = W[:i], up = W[i:]
   cross_entropy_*    == torch.nn.functional.cross_entropy (mean, ignore_index) and its
                      autograd gradient in fp64; rows of the gradient sum to zero
+  adamw_step         == torch.optim.AdamW over several steps in fp64 (parameter and
+                     both moments); with zero gradient only the weight decay acts
   attention_block,   autograd of the composed functions vs. the explicit
   decoder_layer_*    backward formulas in this file
 
@@ -335,6 +337,24 @@ def cross_entropy_fwd_bwd(logits: torch.Tensor, labels: torch.Tensor, ignore_ind
     onehot = torch.zeros_like(p).scatter_(1, safe[:, None], 1.0)
     dlogits = (p - onehot) * valid[:, None].to(ct) * (grad_loss / n)
     return losses.sum() / n, losses, lse, dlogits
+
+
+# --------------------------------------------------------------------------
+# AdamW  (train.py:170,216: torch.optim.AdamW with default betas, eps and weight decay)
+# --------------------------------------------------------------------------
+def adamw_step(param, grad, exp_avg, exp_avg_sq, step: int, lr: float, betas=(0.9, 0.999), eps: float = 1e-8,
+               weight_decay: float = 1e-2):
+    """One decoupled-weight-decay Adam step (Loshchilov & Hutter), as torch.optim.AdamW orders it.
+    Returns the new (param, exp_avg, exp_avg_sq) in the compute dtype."""
+    ct = _ct(param)
+    p, g, m, v = (t.to(ct) for t in (param, grad, exp_avg, exp_avg_sq))
+    b1, b2 = betas
+    p = p * (1.0 - lr * weight_decay)
+    m = b1 * m + (1.0 - b1) * g
+    v = b2 * v + (1.0 - b2) * g * g
+    bc1, bc2 = 1.0 - b1 ** step, 1.0 - b2 ** step
+    p = p - (lr / bc1) * m / (v.sqrt() / (bc2 ** 0.5) + eps)
+    return p, m, v
 
 
 # --------------------------------------------------------------------------

@@ -323,3 +323,22 @@ def test_train_script_accepts_every_mode_of_the_reference():
     from odysseus_transformer_amd.train import parse_args
     for mode in ("odysseus", "ulysses", "dp", "tpsp", "ring"):
         assert parse_args(["--parallel_mode", mode]).parallel_mode == mode
+
+
+def test_adamw_host_side():
+    """Hyper-parameter checks, the parameter-group keys that make its state dicts load into torch.optim.AdamW with the
+    same meaning, and no CPU path."""
+    import pytest as _pytest
+    import torch
+    from odysseus_transformer_amd.optim import AdamW
+    with _pytest.raises(ValueError):
+        AdamW([torch.nn.Parameter(torch.zeros(4))], betas=(1.0, 0.9))
+    p = torch.nn.Parameter(torch.zeros(4))
+    opt = AdamW([p], lr=1e-3)
+    ref = torch.optim.AdamW([torch.nn.Parameter(torch.zeros(4))], lr=1e-3)
+    assert set(ref.param_groups[0]) <= set(opt.param_groups[0])
+    assert opt.param_groups[0]["decoupled_weight_decay"] is True
+    opt.step()                                   # no gradient: nothing happens
+    p.grad = torch.ones(4)
+    with _pytest.raises(RuntimeError, match="no CPU implementation"):
+        opt.step()

@@ -304,3 +304,24 @@ def test_cross_entropy_equals_torch_and_its_autograd():
     assert torch.allclose(losses, torch.nn.functional.cross_entropy(x, y, ignore_index=-100, reduction="none"), rtol=1e-12)
     assert torch.allclose(lse, torch.logsumexp(x, -1))
     assert dx.sum(-1).abs().max() < 1e-12 and (dx[::5] == 0).all()
+
+
+def test_adamw_step_is_torch_adamw():
+    """Parameter and both moments over several steps against torch.optim.AdamW in fp64; zero gradient: decay only."""
+    g = torch.Generator().manual_seed(321)
+    p0 = torch.randn(257, generator=g, dtype=torch.float64)
+    grads = [torch.randn(257, generator=g, dtype=torch.float64) for _ in range(5)]
+    hp = dict(lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    ref = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([ref], **hp)
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step, gr in enumerate(grads, 1):
+        ref.grad = gr.clone()
+        opt.step()
+        p, m, v = oracle.adamw_step(p, gr, m, v, step, **hp)
+        assert torch.allclose(p, ref.detach(), rtol=1e-12, atol=1e-14)
+        assert torch.allclose(m, opt.state[ref]["exp_avg"], rtol=1e-12, atol=1e-14)
+        assert torch.allclose(v, opt.state[ref]["exp_avg_sq"], rtol=1e-12, atol=1e-14)
+    z = torch.zeros_like(p0)
+    p1, m1, v1 = oracle.adamw_step(p0, z, z, z, 1, lr=1e-2, weight_decay=0.5)
+    assert torch.allclose(p1, p0 * (1 - 1e-2 * 0.5)) and not m1.any() and not v1.any()
