@@ -284,15 +284,17 @@ class OdysseusDecoderLayer(nn.Module):
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
 
     def forward(self, hidden_states, attention_mask=None, position_ids=None, **kwargs):
+        # what a host model hands its decoder layers besides (a cache to fill during a prefill)
+        cache = {k: kwargs[k] for k in ("past_key_value", "past_key_values", "cache_position") if kwargs.get(k) is not None}
         if self.fused:
             n1, skip = ops.rmsnorm_fork(hidden_states, self.input_layernorm.weight, self.input_layernorm.variance_epsilon)
-            h = self.self_attn(n1, attention_mask=attention_mask, position_ids=position_ids, residual=skip)[0]
+            h = self.self_attn(n1, attention_mask=attention_mask, position_ids=position_ids, residual=skip, **cache)[0]
             n2, skip = ops.rmsnorm_fork(h, self.post_attention_layernorm.weight,
                                         self.post_attention_layernorm.variance_epsilon)
             return self.mlp(n2, residual=skip)
         residual = hidden_states
         hidden_states = self.self_attn(self.input_layernorm(hidden_states), attention_mask=attention_mask,
-                                       position_ids=position_ids)[0]
+                                       position_ids=position_ids, **cache)[0]
         hidden_states = residual + hidden_states
         residual = hidden_states
         hidden_states = self.mlp(self.post_attention_layernorm(hidden_states))
@@ -308,6 +310,16 @@ def _host_layer_unpacks_two(layer) -> bool:
         return False
 
 
+def _host_layer_returns_tensor(layer) -> bool:
+    """Whether the host's decoder layer returns the hidden states alone (its forward is annotated `-> torch.Tensor`)
+    rather than a tuple that the model unpacks."""
+    try:
+        ann = inspect.signature(layer.forward).return_annotation
+    except (TypeError, ValueError):
+        return False
+    return ann is torch.Tensor or ann in ("torch.Tensor", "Tensor")
+
+
 def _host_builds_no_mask(model) -> None:
     """The modules apply the causal mask themselves and refuse an explicit one.  With the `eager`
     attention implementation transformers hands every layer a dense causal mask; declaring
@@ -321,11 +333,35 @@ def _host_builds_no_mask(model) -> None:
             pass
 
 
-def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True):
+def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True, fuse_layers=False):
     """Swaps every layer's attention (and, by default, MLP) for the Odysseus modules
     (decoder/odysseus.py:298-309).  As in the reference the new modules are freshly
-    initialised: pretrained attention / MLP weights are not carried over."""
+    initialised: pretrained attention / MLP weights are not carried over.
+
+    fuse_layers=True (not in the reference) swaps the whole decoder layer for OdysseusDecoderLayer instead, with
+    the host layer's two norm weights carried over: same arithmetic, but the residual adds ride in the output /
+    down projections' epilogues and the gradient sums at the forks inside the RMSNorm backward.  It needs a host
+    whose decoder layers return the hidden states alone (transformers >= 4.54)."""
     _host_builds_no_mask(model)
+    if fuse_layers:
+        if not use_zero3_linear:
+            raise ValueError("fuse_layers swaps the MLP as well: it needs use_zero3_linear=True")
+        for i in range(model.config.num_hidden_layers):
+            old = model.model.layers[i]
+            if not _host_layer_returns_tensor(old):
+                raise NotImplementedError("this host's decoder layers return tuples: use fuse_layers=False")
+            new = OdysseusDecoderLayer(model.config, i, fused=True).to(model.dtype)
+            new.input_layernorm.weight = old.input_layernorm.weight
+            new.post_attention_layernorm.weight = old.post_attention_layernorm.weight
+            new.input_layernorm.variance_epsilon = getattr(old.input_layernorm, "variance_epsilon", new.input_layernorm.variance_epsilon)
+            new.post_attention_layernorm.variance_epsilon = getattr(old.post_attention_layernorm, "variance_epsilon",
+                                                                    new.post_attention_layernorm.variance_epsilon)
+            for attr in ("attention_type", "gradient_checkpointing"):
+                if hasattr(old, attr):
+                    setattr(new, attr, getattr(old, attr))
+            model.model.layers[i] = new
+        print("Applied Odysseus patch for LlamaDecoderLayer")
+        return
     for i in range(model.config.num_hidden_layers):
         layer = model.model.layers[i]
         new_module = LlamaFlashAttention2TPSP(model.config, i).to(model.dtype)

@@ -55,7 +55,10 @@ def use_native_host_modules(model) -> None:
         new.weight = old.weight
         return new
 
+    from .decoder.odysseus import OdysseusDecoderLayer
     for layer in model.model.layers:
+        if isinstance(layer, OdysseusDecoderLayer):      # already the library's own layer
+            continue
         layer.input_layernorm = native_norm(layer.input_layernorm)
         layer.post_attention_layernorm = native_norm(layer.post_attention_layernorm)
         # the host's own projections (the modes that keep its attention / MLP modules: ulysses, ring, dp)
@@ -117,7 +120,8 @@ def main(args) -> dict:
     if args.parallel_mode == "odysseus":
         print(f"use odysseus zero3 {args.use_ody_zero3}")
         with torch.device(dev):
-            apply_odysseus_attn_patch_llama(model, use_zero3_linear=args.use_ody_zero3)
+            apply_odysseus_attn_patch_llama(model, use_zero3_linear=args.use_ody_zero3,
+                                            fuse_layers=args.fuse_layers and args.use_ody_zero3)
     elif args.parallel_mode == "tpsp":
         with torch.device(dev):
             apply_tpsp_attn_patch_llama(model)
@@ -182,7 +186,8 @@ def main(args) -> dict:
            "step_ms": [round(1e3 * t, 1) for t in step_times], "tokens_per_s": round(args.seq_length * len(step_times) /
                                                                                       max(elapse, 1e-9), 1),
            "peak_memory_gb": round(torch.cuda.max_memory_allocated(dev) / 1024 ** 3, 2), "losses": [round(l, 4) for l in losses],
-           "native_host_modules": bool(args.native_host_modules), "native_optimizer": bool(args.native_optimizer)}
+           "native_host_modules": bool(args.native_host_modules), "native_optimizer": bool(args.native_optimizer),
+           "fuse_layers": bool(args.fuse_layers and args.parallel_mode == "odysseus")}
     print(json.dumps(out))
     return out
 
@@ -201,6 +206,9 @@ def parse_args(argv=None):
     ap.add_argument("--parallel_mode", type=str, choices=["odysseus", "ulysses", "dp", "tpsp", "ring"], default="odysseus")
     ap.add_argument("--num-hidden-layers", type=int, default=16, help="16 in the reference's configuration (train.py:71)")
     ap.add_argument("--native-host-modules", action=argparse.BooleanOptionalAction, default=True)
+    ap.add_argument("--fuse-layers", action=argparse.BooleanOptionalAction, default=True,
+                    help="odysseus mode: swap whole decoder layers (residual adds inside the projections' epilogues) "
+                         "instead of the attention and MLP modules only, as the reference's patch does")
     ap.add_argument("--native-optimizer", action=argparse.BooleanOptionalAction, default=True,
                     help="AdamW as one HIP kernel per tensor instead of torch.optim.AdamW's element-wise passes")
     ap.add_argument("--declare-flash-attention", action=argparse.BooleanOptionalAction, default=False,

@@ -106,9 +106,11 @@ def test_attention_block_unpacked_equals_packed(dev):
     assert rel_err(ya, y_ref) <= TOL_BF16
 
 
-def test_patched_hf_llama_runs_and_matches_oracle(dev):
-    """apply_odysseus_attn_patch_llama on a small transformers Llama: logits and the
-    gradient of the token embedding equal the oracle's composition of the same layers."""
+@pytest.mark.parametrize("fuse_layers", [False, True], ids=["modules_swapped", "layers_swapped"])
+def test_patched_hf_llama_runs_and_matches_oracle(fuse_layers, dev):
+    """apply_odysseus_attn_patch_llama on a small transformers Llama (attention and MLP modules swapped as in the
+    reference, or whole decoder layers): logits and the gradient of the token embedding equal the oracle's
+    composition of the same layers."""
     transformers = pytest.importorskip("transformers")
     from transformers import LlamaConfig, LlamaForCausalLM
     from odysseus_transformer_amd.decoder.odysseus import apply_odysseus_attn_patch_llama
@@ -117,7 +119,8 @@ def test_patched_hf_llama_runs_and_matches_oracle(dev):
                       num_key_value_heads=1, head_dim=128, vocab_size=128, max_position_embeddings=2048,
                       rms_norm_eps=1e-6)
     model = LlamaForCausalLM(cfg).to(torch.bfloat16)
-    apply_odysseus_attn_patch_llama(model)
+    apply_odysseus_attn_patch_llama(model, fuse_layers=fuse_layers)
+    assert type(model.model.layers[0]).__name__ == ("OdysseusDecoderLayer" if fuse_layers else "LlamaDecoderLayer")
     with torch.no_grad():
         for n, prm in model.named_parameters():
             if "mlp" in n or "self_attn" in n:
