@@ -14,7 +14,8 @@ inputs, already resident in HBM).  `value` is the algorithmic TFLOP/s of that st
   tile_cost_ladder  a synthetic kernel of the forward kernel's shape with the ingredients of a tile added one at a
                 time (vector work, LDS operand reads, direct loads), ns per 64-key turn, beside the forward kernel
   configs       the other attention configurations (L = 131072; GQA 4:1 at L = 65536; the ring
-                step over 8 key blocks of 16384): ms, TFLOP/s, % of peak, forward / backward split
+                step over 8 key blocks of 16384; one rank of a zigzag ring of 8): ms, TFLOP/s, % of peak,
+                forward / backward split
   layer         the other pieces of the rank's layer share (QKV / O / MLP GEMMs with
                 torch.matmul on the same tensors as a same-box yardstick, RoPE, RMSNorm, SwiGLU)
                 and the resulting tokens/s as a sum of pieces
@@ -417,6 +418,28 @@ def other_configs(_lib, ops, rn, dev):
     record("cfg5_ring_8x16384", ring_step, 7 * f_full + f_diag, 7 * b_full + b_diag, 5, NB, 2 * NB,
            "ring step through autograd: 16384 queries x 4 heads x 128 against 8 key blocks of 16384 "
            "(block 0 causal), LSE merge after each, backward over all 8")
+    del q, ks, vs, do
+    torch.cuda.empty_cache()
+
+    # one rank of a zigzag ring of 8 (rank 3): its two chunks of 8192 queries against the 8 blocks it would receive,
+    # through autograd; 3 steps see the first chunk of a block with all queries, 4 the whole block with the second chunk
+    c, NR, rank = 8192, 8, 3
+    q = rn((1, 2 * c, H, D), 6000).requires_grad_(True)
+    ks = [rn((1, 2 * c, H, D), 6001 + 2 * b).requires_grad_(True) for b in range(NR)]
+    vs = [rn((1, 2 * c, H, D), 6002 + 2 * b).requires_grad_(True) for b in range(NR)]
+    do = rn((1, 2 * c, H, D), 6100)
+
+    def zigzag_step():
+        for t in [q] + ks + vs:
+            t.grad = None
+        out, _ = ops.zigzag_ring_rank_attn(q, ks, vs, rank, NR)
+        out.backward(do)
+
+    f_c, b_c = attn_flops(2 * c, 2 * c, H, D, causal=True)        # step 0
+    f_r, b_r = attn_flops(2 * c, c, H, D, causal=False)           # every other step: 2c x c or c x 2c score elements
+    record("zigzag_ring_rank3_of_8", zigzag_step, f_c + (NR - 1) * f_r, b_c + (NR - 1) * b_r, 5, NR, 2 * NR,
+           "one rank of a zigzag ring of 8 through autograd: chunks 3 and 12 of a 131072-token sequence (2 x 8192 queries, "
+           "4 heads x 128) against the 8 blocks it receives, LSE merge after each, backward over all 8")
     return res
 
 
