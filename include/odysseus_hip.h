@@ -142,12 +142,20 @@ int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out,
  *                             blocks and rounded once by the caller at the end (ody_cast_from_f32);
  *   ODY_BWD_REUSE_QUERY_SIDE  q, out, lse, dout and the workspace are those of the previous call: delta and
  *                             the other query-side scratch in the workspace are taken as they are (the ring
- *                             step calls once per key block with the same queries).
+ *                             step calls once per key block with the same queries);
+ *   ODY_BWD_KEEP_DS           spends memory to save arithmetic (no counterpart in the reference): the dK/dV
+ *                             kernel keeps dS, rounded to bf16 as it is used there, in the workspace, and dQ is
+ *                             one product dS K over it instead of a second pass over S, dP and dS.  Same
+ *                             results.  For bf16, head_dim 128, causal, Lq == Lk a multiple of 256
+ *                             (ody_attn_bwd_ds_bytes(...) > 0); the workspace then holds
+ *                             ody_attn_bwd_workspace_bytes(...) + ody_attn_bwd_ds_bytes(...) bytes, the latter
+ *                             about B * Hq * Lq * Lq bytes (2 bytes per visible pair).
  * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
  * the bf16 head_dim-128 kernels transposed copies of K, Q and dO).
  */
-enum ody_attn_bwd_flags { ODY_BWD_ACCUMULATE_DQ = 1, ODY_BWD_DQ_F32 = 2, ODY_BWD_REUSE_QUERY_SIDE = 4 };
+enum ody_attn_bwd_flags { ODY_BWD_ACCUMULATE_DQ = 1, ODY_BWD_DQ_F32 = 2, ODY_BWD_REUSE_QUERY_SIDE = 4, ODY_BWD_KEEP_DS = 8 };
 size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
+size_t ody_attn_bwd_ds_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype, int causal);
 int ody_attn_bwd(const void* q, const void* k, const void* v, const void* out, const float* lse,
                  const void* dout, void* dq, void* dk, void* dv,
                  int B, int Lq, int Lk, int Hq, int Hkv, int D,

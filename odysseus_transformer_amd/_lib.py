@@ -13,7 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libodysseus_hip.so"
 
 ODY_BF16, ODY_F32 = 0, 1
 GEMM_NT, GEMM_NN, GEMM_TN = 0, 1, 2
-BWD_ACCUMULATE_DQ, BWD_DQ_F32, BWD_REUSE_QUERY_SIDE = 1, 2, 4
+BWD_ACCUMULATE_DQ, BWD_DQ_F32, BWD_REUSE_QUERY_SIDE, BWD_KEEP_DS = 1, 2, 4, 8
 ATTN_FWD_NOALLOC_SCRATCH_BYTES = (32 << 20) + (64 << 10)
 
 _i, _i64, _f, _p, _sz = C.c_int, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
@@ -31,6 +31,7 @@ SIGNATURES = {
     "ody_attn_fwd": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p, _sz, _p]),
     "ody_attn_fwd_noalloc": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p]),
     "ody_attn_bwd_workspace_bytes": (_sz, [_i] * 7),
+    "ody_attn_bwd_ds_bytes": (_sz, [_i] * 8),
     "ody_attn_bwd": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p]),
     "ody_cast_from_f32": (_i, [_p, _p, _i64, _i, _p]),
     "ody_lse_merge": (_i, [_p] * 4 + [_i] * 4 + [_i64] * 3 + [_i, _p]),

@@ -134,6 +134,11 @@ extern "C" size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, in
   return n;
 }
 
+extern "C" size_t ody_attn_bwd_ds_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype, int causal) {
+  if (B <= 0 || Lq <= 0 || Lk <= 0 || Hq <= 0 || Hkv <= 0 || dtype != ODY_BF16 || D != 128) return 0;
+  return (ody_attn_bwd_pipe_ds_bytes(B, Lq, Lk, Hq, causal) + 255) & ~(size_t)255;
+}
+
 namespace {
 int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
                   const void* q, const void* k, const void* v, const void* out, const float* lse,
@@ -151,7 +156,7 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
                   void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common(who, B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
-  ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE)) == 0, ODY_ERR_UNSUPPORTED,
+  ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE | ODY_BWD_KEEP_DS)) == 0, ODY_ERR_UNSUPPORTED,
               "%s: unknown flag bits in %d", who, flags);
   AttnParams p{};
   p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
@@ -176,9 +181,15 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
   ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "%s: lse is NULL", who);
   ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "%s: scale must be positive", who);
   ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "%s: workspace is NULL", who);
-  ODY_REQUIRE(workspace_bytes >= ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype), ODY_ERR_WORKSPACE,
-              "%s: workspace of %zu bytes, %zu needed", who, workspace_bytes,
-              ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype));
+  const size_t ws_base = ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype);
+  size_t ws_ds = 0;
+  if (flags & ODY_BWD_KEEP_DS) {
+    ws_ds = ody_attn_bwd_ds_bytes(B, Lq, Lk, Hq, Hkv, D, dtype, causal);
+    ODY_REQUIRE(ws_ds > 0, ODY_ERR_UNSUPPORTED,
+                "%s: ODY_BWD_KEEP_DS needs bf16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256", who);
+  }
+  ODY_REQUIRE(workspace_bytes >= ws_base + ws_ds, ODY_ERR_WORKSPACE, "%s: workspace of %zu bytes, %zu needed", who,
+              workspace_bytes, ws_base + ws_ds);
   ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
               "%s: workspace must be 256-byte aligned", who);
   if (rope_q || rope_k) {
@@ -191,6 +202,7 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
     p.rope_k = static_cast<const bf16*>(rope_k);
   }
   p.delta = static_cast<float*>(workspace);
+  if (ws_ds) p.ds = reinterpret_cast<bf16*>(static_cast<char*>(workspace) + ws_base);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == ODY_BF16 && D == 128)   // its query-side pre-pass computes delta as well
     return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);

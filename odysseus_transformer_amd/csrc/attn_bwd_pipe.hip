@@ -26,6 +26,61 @@ using namespace tile128;
 constexpr int D = 128, KS = D / 16, DT = D / 32;
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// dQ^T of one query held by lane group g (accumulator rows 8 (r >> 2) + 4 g + (r & 3) of each 32-wide slice of the
+// head dimension) -> row qi of dq: scaled, then added to an fp32 or bf16 destination, rotated back by the rotary
+// table, or rounded and stored.
+__device__ __forceinline__ void store_dq_row(const AttnParams& p, const f32x16 (&dq)[DT], int b, int h, int qi, int g) {
+  if (qi >= p.Lq) return;
+  if (p.dq_f32) {
+    // fp32 destination (the ring step's running dq): exact accumulation over the key blocks, no rounding here
+    float* dqp = static_cast<float*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        f32x4* dst = reinterpret_cast<f32x4*>(dqp + 32 * dt + 8 * a + 4 * g);
+        f32x4 w = {0.f, 0.f, 0.f, 0.f};
+        if (p.accumulate_dq) w = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] += dq[dt][4 * a + e] * p.scale;
+        *dst = w;
+      }
+  } else if (p.rope_q) {
+    // the gradient of the un-rotated projection: element d < 64 pairs with d + 64, both in this lane
+    bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+    const bf16* trow = p.rope_q + ((int64_t)b * p.Lq + qi) * D;
+#pragma unroll
+    for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        const bf16x8 cs = *reinterpret_cast<const bf16x8*>(trow + 2 * (32 * dt + 8 * a + 4 * g));
+        bf16x4 w1, w2;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+          const float g1 = dq[dt][4 * a + e] * p.scale, g2 = dq[dt + 2][4 * a + e] * p.scale;
+          w1[e] = (bf16)(g1 * c + g2 * sn);
+          w2[e] = (bf16)(g2 * c - g1 * sn);
+        }
+        *reinterpret_cast<bf16x4*>(dqp + 32 * dt + 8 * a + 4 * g) = w1;
+        *reinterpret_cast<bf16x4*>(dqp + 32 * (dt + 2) + 8 * a + 4 * g) = w2;
+      }
+  } else {
+    bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        bf16x4* dst = reinterpret_cast<bf16x4*>(dqp + 32 * dt + 8 * a + 4 * g);
+        bf16x4 w, old = {0, 0, 0, 0};
+        if (p.accumulate_dq) old = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = (bf16)(dq[dt][4 * a + e] * p.scale + (float)old[e]);
+        *dst = w;
+      }
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------
@@ -202,58 +257,7 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
     if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 1);
   }
 
-#pragma unroll
-  for (int qt = 0; qt < QT; qt++) {
-    const int qi = wq0 + 32 * qt + i;
-    if (qi < p.Lq && p.dq_f32) {
-      // fp32 destination (the ring step's running dq): exact accumulation over the key blocks, no rounding here
-      float* dqp = static_cast<float*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
-#pragma unroll
-      for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-          f32x4* dst = reinterpret_cast<f32x4*>(dqp + 32 * dt + 8 * a + 4 * g);
-          f32x4 w = {0.f, 0.f, 0.f, 0.f};
-          if (p.accumulate_dq) w = *dst;
-#pragma unroll
-          for (int e = 0; e < 4; e++) w[e] += dq[qt][dt][4 * a + e] * p.scale;
-          *dst = w;
-        }
-    } else if (qi < p.Lq && p.rope_q) {
-      // the gradient of the un-rotated projection: element d < 64 pairs with d + 64, both in this lane
-      bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
-      const bf16* trow = p.rope_q + ((int64_t)b * p.Lq + qi) * D;
-#pragma unroll
-      for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-          const bf16x8 cs = *reinterpret_cast<const bf16x8*>(trow + 2 * (32 * dt + 8 * a + 4 * g));
-          bf16x4 w1, w2;
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
-            const float g1 = dq[qt][dt][4 * a + e] * p.scale, g2 = dq[qt][dt + 2][4 * a + e] * p.scale;
-            w1[e] = (bf16)(g1 * c + g2 * sn);
-            w2[e] = (bf16)(g2 * c - g1 * sn);
-          }
-          *reinterpret_cast<bf16x4*>(dqp + 32 * dt + 8 * a + 4 * g) = w1;
-          *reinterpret_cast<bf16x4*>(dqp + 32 * (dt + 2) + 8 * a + 4 * g) = w2;
-        }
-    } else if (qi < p.Lq) {
-      bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l;
-#pragma unroll
-      for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-          bf16x4* dst = reinterpret_cast<bf16x4*>(dqp + 32 * dt + 8 * a + 4 * g);
-          bf16x4 w, old = {0, 0, 0, 0};
-          if (p.accumulate_dq) old = *dst;
-#pragma unroll
-          for (int e = 0; e < 4; e++) w[e] = (bf16)(dq[qt][dt][4 * a + e] * p.scale + (float)old[e]);
-          *dst = w;
-        }
-    }
-  }
+  store_dq_row(p, dq[0], b, h, wq0 + i, g);
 }
 
 // ---------------------------------------------------------------------------------
@@ -271,6 +275,20 @@ constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 *
 constexpr int KV_STAT_ELEMS = 128 * 8;                                   // start-value fragments of one tile
 constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q, dO tiles; Q^T, dO^T images; start values
 
+// dS kept for the dQ kernel (causal, Lq == Lk, a multiple of 256): one 128 KB block per (256-key block kb, 256-query
+// block qb >= kb), laid out for the reader, which takes 64 keys x 256 queries at a time:
+//   [64-key tile y = 0..3][64-query tile x = 0..3][chunk c = 0..7][key 0..63][8 bf16]
+// Element j of chunk c is the query of tile row 32 (j >> 2) + 16 (c & 1) + 4 (j & 3) + ((c >> 1) & 1) + 2 (c >> 2) -- the
+// order in which an accumulator holds the rows, i.e. image_pos(row) = 8 c + j.  Blocks of one (batch, head) are
+// contiguous, key block after key block, and inside a key block by qb.  Entries of masked pairs are 0; the parts
+// (y, x) of a diagonal block with y > x, whose keys all come after their queries, are never written (and never used).
+constexpr int DS_PIECE = 64 * 8;                 // one (y, x, c): 1 KB
+constexpr int DS_BLOCK_ELEMS = 4 * 4 * 8 * DS_PIECE;
+__host__ __device__ inline int64_t ds_blocks_per_head(int nb) { return (int64_t)nb * (nb + 1) / 2; }
+__host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
+  return (int64_t)kb * nb - (int64_t)kb * (kb - 1) / 2 + (qb - kb);
+}
+
 // The start values of S and dP for every 64-query tile enter as one more A-operand fragment of the contraction
 // (the matching B fragment is all ones): the fp32 value x is split into three bf16 terms x = h + m + l, which
 // the MFMA adds up exactly like any other product.  The query-side pre-pass (attn_bwd_prepass_kernel) writes
@@ -281,7 +299,11 @@ constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q,
 // SPLIT = true (grouped-query attention): a block owns 256 keys for ONE query head and writes
 // fp32 partial dK / dV to `part`, which attn_bwd_group_sum_kernel adds up over the group.  With few
 // kv heads this is what gives the chip enough, and evenly sized, blocks.
-template <bool SPLIT>
+//
+// KEEP_DS = true (causal self-attention, Lq == Lk a multiple of 256): every dS tile also goes to p.ds, in the
+// layout described at ds_block_index, and the dQ kernel below (attn_bwd_dq_from_ds_kernel) reads it back
+// instead of computing S, dP and dS a second time.
+template <bool SPLIT, bool KEEP_DS>
 __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
                                                                          const bf16* __restrict__ qimg,
                                                                          const bf16* __restrict__ doimg,
@@ -360,7 +382,9 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 
   // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
   // work, 16 MFMAs for dV^T and dK^T
-  auto sub_tile = [&](const bf16* st, int t, int mt, bool masked) {
+  // kept dS: chunk 4 mt + 2 ss + g of part (y, x) = (wave >> 1, t & 3) of the block, to which `tile` points at this
+  // wavefront's 32 keys.  Streaming stores: the tiles are read once, by another kernel.
+  auto sub_tile = [&](const bf16* st, int t, int mt, bool masked, bf16* ds_tile) {
     const int ln = fresh_lane(), g = ln >> 5, i = ln & 31;
     const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
     const bf16* Qt = st;
@@ -410,10 +434,21 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
       pf[r >> 3][r & 7] = (bf16)pr;
       dsf[r >> 3][r & 7] = (bf16)(pr * dp[r]);
     }
+    // Kept dS: dsf[ss] is chunk 4 mt + 2 ss + g of this lane's key, 512 contiguous bytes per half wavefront;
+    // ds_tile points at part (y, x) = (wave >> 1, t & 3) of the block, at this wavefront's 32 keys.  Streaming
+    // stores (the tiles are read once, by another kernel), one under each half of the MFMAs below.  (Holding them
+    // back in LDS until the next sub-tile, so that none is still on its way at the top of the next iteration, where
+    // the wait for the tile loads waits for stores as well, was measured slower.)
+    auto keep = [&](int ss) {
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+      u32x4* dst = reinterpret_cast<u32x4*>(ds_tile + (unsigned)((4 * mt + 2 * ss + g) * DS_PIECE + i * 8));
+      __builtin_nontemporal_store(__builtin_bit_cast(u32x4, dsf[ss]), dst);
+    };
     FENCE();
 #pragma unroll
     for (int n = 0; n < 8; n++) {
       const int dt = n & 3, ss = n >> 2;
+      if (KEEP_DS && (n == 1 || n == 5)) keep(n >> 2);
       dv[dt] = mfma32(oif[n % PF], pf[ss], dv[dt]);
       dk[dt] = mfma32(qif[n % PF], dsf[ss], dk[dt]);
       if (n + PF < 8) {
@@ -433,12 +468,18 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     // every query of the tile is before every key of this wavefront: nothing to do
     const bool dead = p.causal && (t * KV_BQ + KV_BQ - 1 + p.off < wn0);
     const bool masked = p.causal && (t * KV_BQ + p.off < wn0 + 31);
+    bf16* ds_tile = nullptr;
+    if (KEEP_DS) {
+      const int nb = q_tiles / 4;
+      ds_tile = p.ds + (((int64_t)b * p.Hq + h_first + it / ntq) * ds_blocks_per_head(nb) + ds_block_index(nb, bc.rank, t >> 2)) * DS_BLOCK_ELEMS +
+                (((wave >> 1) * 4 + (t & 3)) * 8) * DS_PIECE + (wave & 1) * 32 * 8;
+    }
 #pragma unroll 1
     for (int mt = 0; mt < 2; mt++) {
       // the loads of the next stage go out in two halves, one before each sub-tile: issued all at
       // once by eight wavefronts they would queue up behind each other at the memory pipeline
       if (it + 1 < total) load_stage(ring + ((it + 1) & 1) * KV_STAGE, it + 1, mt);
-      if (!dead) sub_tile(st, t, mt, masked);
+      if (!dead) sub_tile(st, t, mt, masked, ds_tile);
     }
   }
 
@@ -502,6 +543,113 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   }
 }
 
+// ---------------------------------------------------------------------------------
+// dQ from the kept dS
+// ---------------------------------------------------------------------------------
+// One product, dQ^T += K^T dS^T, over the tiles that the dK/dV kernel (KEEP_DS) left in p.ds.  256 queries per block,
+// 8 wavefronts x 32 queries: wavefront w owns chunks 4 (w & 1) ... + 3 of 64-query tile (w >> 1) of the block, lane i
+// the query at position 32 (w & 1) + i of that tile's kept order.  A three-deep ring of {the 32 one-KB pieces of dS
+// that belong to this 64-key tile and the block's 4 query tiles, K^T image}.
+//
+//      A: K^T image (LDS, 16-byte reads), as in the dQ kernel above
+//      B: dS^T.  The tiles hold 8 queries of one key side by side, the product contracts over keys: the transposing
+//         LDS read turns 4 keys x 16 queries into 4-key pieces per query, two of them make a fragment.
+//
+// 2 bytes per visible (query, key) pair for 256 flops: the kernel is bound by HBM, half of the matrix pipe idles.
+constexpr int DS_PIECE_ELEMS = GROUP_ELEMS;   // 1 KB + 16 bytes: consecutive pieces start 4 banks apart
+constexpr int DQS_STAGE = 32 * DS_PIECE_ELEMS + IMG_ELEMS;
+
+__global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_from_ds_kernel(const AttnParams p,
+                                                                          const bf16* __restrict__ kimg) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* ring = reinterpret_cast<bf16*>(smem_raw);     // [3][DQS_STAGE]
+
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
+            i = lane & 31;
+  const BlockCoord bc = ody_block_coord(p.Hq, p.B);
+  const int nqb = gridDim.x / (p.Hq * p.B);
+  const int qblk = nqb - 1 - bc.rank;   // heaviest blocks first
+  const int h = bc.h, b = bc.b, hk = h / p.group;
+  const int q_tiles = p.Lq / KV_BQ, x = wave >> 1, mt = wave & 1;
+  const bf16* kip = kimg + ((int64_t)b * p.Hkv + hk) * (p.Lk / 64) * IMG_ELEMS;
+  const int nb = q_tiles / 4;
+  const bf16* dsh = p.ds + ((int64_t)b * p.Hq + h) * ds_blocks_per_head(nb) * DS_BLOCK_ELEMS;
+  const int ntiles = 4 * (qblk + 1);   // 64-key tiles up to the block's last query
+
+  auto load_part = [&](bf16* st, int t, int j) {   // j = 0, 1: the two halves of a stage's loads
+    // the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk): 32 KB in a row
+    const bf16* src = dsh + ds_block_index(nb, t >> 2, qblk) * DS_BLOCK_ELEMS + (t & 3) * (32 * DS_PIECE);
+#pragma unroll
+    for (int n = 0; n < 2; n++) {
+      const int piece = 8 * (2 * j + n) + wave;   // query tile 2 j + n of the block, chunk `wave`
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (unsigned)(piece * DS_PIECE + lane * 8)),
+                                       (lds_void_ptr)(st + piece * DS_PIECE_ELEMS), 16, 0, 0);
+    }
+    const int grp = DQ_WAVES * j + wave;
+    __builtin_amdgcn_global_load_lds((global_void_ptr)(kip + (int64_t)t * IMG_ELEMS + (grp * 64 + lane) * 8),
+                                     (lds_void_ptr)(st + 32 * DS_PIECE_ELEMS + grp * 512), 16, 0, 0);
+  };
+  load_part(ring, 0, 0);
+  load_part(ring, 0, 1);
+  load_part(ring + DQS_STAGE, 1, 0);   // ntiles >= 4
+  load_part(ring + DQS_STAGE, 1, 1);
+
+  f32x16 dq[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dq[dt][r] = 0.f;
+
+  const int ibase = image_frag_base(g, i);
+  // the transposing read: inside 16 lanes, lane 4 k + m supplies key 4 k (+ the fragment's row offset) and queries
+  // 4 m ... 4 m + 3 of the 16; queries 0-7 of the 16 are one chunk, 8-15 the next
+  const int sbase = (8 * x + 4 * mt + 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) * DS_PIECE_ELEMS +
+                    (16 * g + 4 * ((lane >> 2) & 3)) * 8 + 4 * (lane & 1);
+
+  auto tile = [&](const bf16* st) {
+    const bf16* Sp = st + sbase;
+    const bf16* Ki = st + 32 * DS_PIECE_ELEMS;
+    constexpr int IPF = 4;
+    bf16x8 ifr[IPF], dsf[2][2];
+#pragma unroll
+    for (int n = 0; n < IPF; n++) ifr[n] = image_frag(Ki, ibase, n & 3, 0, 0);
+#pragma unroll
+    for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+      for (int ss = 0; ss < 2; ss++)   // keys 32 (j >> 2) + 16 g + 4 (j & 3) + ss + 2 kt, j = 0..7
+        dsf[kt][ss] = concat4(lds_read_tr16(Sp + (ss + 2 * kt) * 8), lds_read_tr16(Sp + (ss + 2 * kt) * 8 + 32 * 8));
+    FENCE();
+#pragma unroll
+    for (int n = 0; n < 16; n++) {
+      const int dt = n & 3, ss = (n >> 2) & 1, kt = n >> 3;
+      dq[dt] = mfma32(ifr[n % IPF], dsf[kt][ss], dq[dt]);
+      if (n + IPF < 16) {
+        const int m = n + IPF;
+        ifr[n % IPF] = image_frag(Ki, ibase, m & 3, (m >> 2) & 1, m >> 3);
+      }
+      FENCE();
+    }
+  };
+
+  for (int t = 0; t < ntiles; t++) {
+    // stage t landed (the loads of stage t+1 may still be in flight), everyone done with stage t-1
+    if (t + 1 < ntiles) {
+      asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    // the loads go first: what bounds this kernel is the time a tile spends on its way from HBM, and issued here
+    // a tile has two iterations to arrive
+    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * DQS_STAGE, t + 2, 0);
+    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * DQS_STAGE, t + 2, 1);
+    // tiles whose keys all come after this wavefront's queries were never written
+    if (t <= 4 * qblk + x) tile(ring + (t % 3) * DQS_STAGE);
+  }
+
+  // position 32 mt + i of the tile's kept order = chunk 4 mt + (i >> 3), element i & 7
+  const int row = 32 * ((i >> 2) & 1) + 16 * ((i >> 3) & 1) + 4 * (i & 3) + (i >> 4) + 2 * mt;
+  store_dq_row(p, dq, b, h, qblk * DQ_BM + KV_BQ * x + row, g);
+}
+
 // dK, dV of a kv head = sum of the fp32 partials of its query heads; one thread per 4 elements d..d+3 of the first half
 // of a key row and their partners d + 64 (the pairs of the rotary embedding)
 __global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParams p, const float* __restrict__ part) {
@@ -561,12 +709,22 @@ size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
          group_partials_bytes(B, Lk, Hq, Hkv);
 }
 
+size_t ody_attn_bwd_pipe_ds_bytes(int B, int Lq, int Lk, int Hq, int causal) {
+  if (!causal || Lq != Lk || Lq % KV_BN != 0 || B <= 0 || Hq <= 0) return 0;
+  return (size_t)B * Hq * ds_blocks_per_head(Lq / KV_BN) * DS_BLOCK_ELEMS * sizeof(bf16);
+}
+
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem_q = (size_t)3 * (2 * TILE_ELEMS + IMG_ELEMS) * sizeof(bf16);
   constexpr size_t smem_kv = (size_t)2 * KV_STAGE * sizeof(bf16);
+  constexpr size_t smem_qs = (size_t)3 * DQS_STAGE * sizeof(bf16);
+  static_assert(smem_qs <= 160 * 1024, "LDS of one CU");
   for (const auto& ks : {std::pair<const void*, size_t>{reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel), smem_q},
-                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false>), smem_kv},
-                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true>), smem_kv}})
+                         {reinterpret_cast<const void*>(&attn_bwd_dq_from_ds_kernel), smem_qs},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false, false>), smem_kv},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true, false>), smem_kv},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false, true>), smem_kv},
+                         {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true, true>), smem_kv}})
     if (int rc = ody_allow_dynamic_lds(ks.first, ks.second, "attn_bwd")) return rc;
   unsigned char* w = static_cast<unsigned char*>(workspace);
   bf16* kimg = reinterpret_cast<bf16*>(w);
@@ -581,15 +739,23 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
   const int key_blocks = (p.Lk + KV_BN - 1) / KV_BN;
   if (p.group == 1) {
-    ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<false>, dim3(key_blocks * p.Hkv * p.B),
-               dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
+    if (p.ds)
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<false, true>), dim3(key_blocks * p.Hkv * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
+    else
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<false, false>), dim3(key_blocks * p.Hkv * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
     if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
   } else {
     float* part = reinterpret_cast<float*>(
         reinterpret_cast<unsigned char*>(stats) +
         align256((size_t)p.B * p.Hq * ((p.Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)));
-    ODY_LAUNCH("attn_bwd_dkdv_pipe", st, attn_bwd_dkdv_pipe_kernel<true>, dim3(key_blocks * p.Hq * p.B),
-               dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
+    if (p.ds)
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, true>), dim3(key_blocks * p.Hq * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
+    else
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, false>), dim3(key_blocks * p.Hq * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
     if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
     const int64_t n8 = (int64_t)p.B * p.Hkv * p.Lk * (D / 8);
     ODY_LAUNCH("attn_bwd_group_sum", st, attn_bwd_group_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p,
@@ -597,6 +763,13 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
     if ((rc = ody_check_launch("attn_bwd_group_sum"))) return rc;
   }
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
+  if (p.ds) {
+    // what ody_attn_bwd_pipe_ds_bytes promised: whole 256-row blocks on both sides, queries and keys aligned
+    ODY_REQUIRE(p.causal && p.off == 0 && p.Lq % KV_BN == 0 && KV_BN == DQ_BM, ODY_ERR_UNSUPPORTED,
+                "attn_bwd: kept dS needs causal self-attention on a multiple of %d rows", KV_BN);
+    ODY_LAUNCH("attn_bwd_dq_from_ds", st, attn_bwd_dq_from_ds_kernel, gq, dim3(DQ_THREADS), smem_qs, p, kimg);
+    return ody_check_launch("attn_bwd_dq_from_ds");
+  }
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");
 }

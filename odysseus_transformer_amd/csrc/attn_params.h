@@ -28,6 +28,9 @@ struct AttnParams {
   // gradient of the projection BEFORE its rotary embedding
   const bf16* rope_q;
   const bf16* rope_k;
+  // bwd, bf16 head_dim 128, causal self-attention with Lq == Lk a multiple of 256: when set, the dK/dV kernel keeps
+  // every dS tile here (ody_attn_bwd_ds_bytes) and dQ is computed from them instead of from a second pass over S and dP
+  bf16* ds;
   float scale;        // softmax scale
   float scale_log2e;  // scale * log2(e)
   AttnStrides sq, sk, sv, so, sdo, sdq, sdk, sdv;
@@ -65,6 +68,8 @@ size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
 int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st);
 // head_dim 128 only; workspace of ody_attn_bwd_pipe_workspace(...) bytes (p.delta is set separately)
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
+// bytes of the kept dS tiles (AttnParams::ds), 0 where the shape does not qualify
+size_t ody_attn_bwd_pipe_ds_bytes(int B, int Lq, int Lk, int Hq, int causal);
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st);
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st);
 // fp32 on the fp32 matrix cores

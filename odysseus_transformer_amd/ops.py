@@ -7,6 +7,7 @@ is the only compute path.
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -111,14 +112,20 @@ def attn_fwd_noalloc(q, k, v, out, lse, causal: bool = True, scale: Optional[flo
 
 def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
              dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False,
-             rope_tables=None):
+             rope_tables=None, keep_ds: Optional[bool] = None):
     """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.
 
     dq may be a float32 tensor although q is bfloat16: with accumulate_dq that is the running dq of a
     ring step, summed exactly over the key blocks.  reuse_query_side=True (needs the `workspace` of
     the previous call, with the same q / out / lse / dout) skips the scratch that depends on the
     queries only.  rope_tables=(table_q, table_k) (rope_table() of the query / key positions; bf16,
-    head_dim 128) makes dq and dk the gradients of the projection BEFORE its rotary embedding."""
+    head_dim 128) makes dq and dk the gradients of the projection BEFORE its rotary embedding.
+
+    keep_ds spends scratch memory to save arithmetic: the dK/dV kernel keeps dS (2 bytes per visible
+    query-key pair, about B * Hq * L * L bytes) and dQ becomes one product over it instead of a second
+    pass over S and dP.  bfloat16, head_dim 128, causal, Lq == Lk a multiple of 256 only.  None (the
+    default) turns it on where the shape qualifies, no `workspace` is passed and the scratch stays within
+    keep_ds_max_bytes(); True insists (ValueError where the shape does not qualify); False never."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
@@ -138,16 +145,30 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     lib = _lib.load()
     ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
+    ds_bytes = lib.ody_attn_bwd_ds_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q), int(causal)) if keep_ds is not False else 0
+    if keep_ds and ds_bytes == 0:
+        raise ValueError("keep_ds needs bfloat16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256")
+    ws = None
+    if keep_ds is None:
+        keep_ds = workspace is None and 0 < ds_bytes <= keep_ds_max_bytes(q.device)
+        if keep_ds:
+            try:
+                ws = scratch(ws_bytes + ds_bytes, "attn_bwd_workspace", q.device)
+            except torch.OutOfMemoryError:   # the memory is not there: the recomputing kernels need none of it
+                keep_ds = False
+    if keep_ds:
+        ws_bytes += ds_bytes
     if workspace is None:
         if reuse_query_side:
             raise ValueError("reuse_query_side needs the workspace of the previous call")
-        ws = scratch(ws_bytes, "attn_bwd_workspace", q.device)
+        if ws is None:
+            ws = scratch(ws_bytes, "attn_bwd_workspace", q.device)
     else:
         ws = workspace
         if ws.dtype != torch.uint8 or ws.numel() < ws_bytes or ws.device != q.device or not ws.is_contiguous():
             raise ValueError(f"workspace must be a contiguous uint8 tensor of at least {ws_bytes} bytes on {q.device}")
     flags = (_lib.BWD_ACCUMULATE_DQ if accumulate_dq else 0) | (_lib.BWD_DQ_F32 if dq_f32 else 0) | \
-            (_lib.BWD_REUSE_QUERY_SIDE if reuse_query_side else 0)
+            (_lib.BWD_REUSE_QUERY_SIDE if reuse_query_side else 0) | (_lib.BWD_KEEP_DS if keep_ds else 0)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise ValueError("lse must be a contiguous float32 tensor (B, Hq, Lq)")
     args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
@@ -167,10 +188,37 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     return dq, dk, dv
 
 
-def attn_bwd_workspace(q, k) -> torch.Tensor:
-    """A workspace for attn_bwd on these shapes, for callers that make several calls with the same queries."""
+_KEEP_DS_MAX_BYTES: Optional[int] = None
+
+
+def keep_ds_max_bytes(device=None) -> int:
+    """Largest dS scratch that attn_bwd takes on its own (keep_ds=None): set_keep_ds_max_bytes(), else the
+    environment variable ODYSSEUS_KEEP_DS_MAX_BYTES, else a quarter of the device's memory."""
+    if _KEEP_DS_MAX_BYTES is not None:
+        return _KEEP_DS_MAX_BYTES
+    env = os.environ.get("ODYSSEUS_KEEP_DS_MAX_BYTES")
+    if env is not None:
+        return int(env)
+    return torch.cuda.get_device_properties(device).total_memory // 4
+
+
+def set_keep_ds_max_bytes(nbytes: Optional[int]) -> None:
+    """0 turns the automatic use of keep_ds off; None restores the default."""
+    global _KEEP_DS_MAX_BYTES
+    _KEEP_DS_MAX_BYTES = nbytes
+
+
+def attn_bwd_workspace(q, k, keep_ds: bool = False, causal: bool = True) -> torch.Tensor:
+    """A workspace for attn_bwd on these shapes, for callers that make several calls with the same queries
+    (keep_ds: with room for the kept dS of attn_bwd(..., keep_ds=True))."""
     B, Lq, Hq, D = q.shape
-    n = _lib.load().ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q))
+    lib = _lib.load()
+    n = lib.ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q))
+    if keep_ds:
+        ds = lib.ody_attn_bwd_ds_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q), int(causal))
+        if ds == 0:
+            raise ValueError("keep_ds needs bfloat16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256")
+        n += ds
     return torch.empty(n, dtype=torch.uint8, device=q.device)
 
 

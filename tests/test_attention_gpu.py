@@ -201,3 +201,82 @@ def test_attention_random_shapes_fp32(case, D, dev):
     assert_parity(dq - dq0, dq_ref, 4 * TOL_F32, "dq", floor)  # the difference of two rounded sums
     assert_parity(dk, dk_ref, TOL_F32, "dk", floor)
     assert_parity(dv, dv_ref, TOL_F32, "dv")
+
+
+KEEP_DS_CASES = [
+    # B, L, Hq, Hkv
+    (1, 256, 1, 1),
+    (2, 512, 2, 2),      # batch 2: the tiles of every (batch, head) are their own region
+    (1, 768, 4, 1),      # GQA 4:1: the dK/dV kernel writes per-query-head partials
+    (1, 1280, 4, 2),     # 5 blocks: an odd number of 256-row blocks
+]
+
+
+@pytest.mark.parametrize("keep_ds", [False, True], ids=["recompute", "keep_ds"])
+@pytest.mark.parametrize("case", KEEP_DS_CASES, ids=lambda c: "B%d_L%d_H%d_%d" % c)
+def test_attention_bwd_kept_ds(case, keep_ds, dev):
+    """dQ as one product over the dS tiles that the dK/dV kernel keeps, against the oracle -- and the recomputing
+    kernels on the same shapes, which the default setting no longer takes there."""
+    from odysseus_transformer_amd import ops
+    B, L, Hq, Hkv = case
+    print(f"case={case} keep_ds={keep_ds}", flush=True)
+    q, k, v, do = _inputs(B, L, L, Hq, Hkv, 128, torch.bfloat16, seed=L + Hq)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=True)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float(), causal=True)
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=True)
+    dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True, keep_ds=keep_ds)
+    assert_parity(dq, dq_ref, TOL_BF16, "dq", 1e-3)
+    assert_parity(dk, dk_ref, TOL_BF16, "dk", 1e-3)
+    assert_parity(dv, dv_ref, TOL_BF16, "dv")
+    # the same dq through the other destinations of the epilogue: an fp32 running sum, a bf16 one, the rotary tables
+    acc0 = randn((B, L, Hq, 128), 5).to(dev)
+    acc = acc0.clone()
+    ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True, dq=acc, accumulate_dq=True, keep_ds=keep_ds)
+    assert_parity((acc - acc0).cpu(), dq_ref, TOL_BF16, "dq added to an fp32 buffer", 1e-3)
+    accb = acc0.to(torch.bfloat16)
+    ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True, dq=accb, accumulate_dq=True, keep_ds=keep_ds)
+    assert_parity(accb, acc0.to(torch.bfloat16).float().cpu() + dq_ref, TOL_BF16, "dq added to a bf16 buffer")
+    pos = torch.arange(L, device=dev).repeat(B, 1)
+    table = ops.rope_table(pos, B * L, 128, 10000.0)
+    dq_r, dk_r, _ = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=True, rope_tables=(table, table), keep_ds=keep_ds)
+    cos, sin = oracle.rope_cos_sin(pos.cpu(), 128, 10000.0)
+    assert_parity(dq_r, oracle.apply_rope_bwd(dq_ref, cos, sin), TOL_BF16, "dq rotated back", 1e-3)
+    assert_parity(dk_r, oracle.apply_rope_bwd(dk_ref, cos, sin), TOL_BF16, "dk rotated back", 1e-3)
+
+
+def test_attention_bwd_kept_ds_policy(dev):
+    """keep_ds=None takes the kept-dS kernels where the shape qualifies and the scratch fits the limit; True on a
+    shape that does not qualify is an error; the C ABI refuses a workspace without room for dS."""
+    from odysseus_transformer_amd import ops, _lib
+    lib = _lib.load()
+    assert lib.ody_attn_bwd_ds_bytes(1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 1) == 2 * 3 * 128 * 1024
+    for args in ((1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 0), (1, 500, 500, 2, 2, 128, _lib.ODY_BF16, 1),
+                 (1, 512, 768, 2, 2, 128, _lib.ODY_BF16, 1), (1, 512, 512, 2, 2, 64, _lib.ODY_BF16, 1),
+                 (1, 512, 512, 2, 2, 128, _lib.ODY_F32, 1)):
+        assert lib.ody_attn_bwd_ds_bytes(*args) == 0, args
+    q, k, v, do = (t.to(dev) for t in _inputs(1, 512, 512, 2, 2, 128, torch.bfloat16, seed=3))
+    o, lse = ops.attn_fwd(q, k, v, causal=True)
+
+    def kernels(**kw):
+        _lib.profile_enable(True)
+        try:
+            ops.attn_bwd(q, k, v, o, lse, do, causal=True, **kw)
+            torch.cuda.synchronize()
+            return set(_lib.profile_collect())
+        finally:
+            _lib.profile_enable(False)
+
+    assert "attn_bwd_dq_from_ds" in kernels()
+    ops.set_keep_ds_max_bytes(0)
+    try:
+        assert "attn_bwd_dq_pipe" in kernels()
+        assert "attn_bwd_dq_from_ds" in kernels(keep_ds=True)
+    finally:
+        ops.set_keep_ds_max_bytes(None)
+    with pytest.raises(ValueError):
+        ops.attn_bwd(q[:, :500], k[:, :500], v[:, :500], o[:, :500], lse[:, :, :500].contiguous(), do[:, :500],
+                     causal=True, keep_ds=True)
+    small = ops.attn_bwd_workspace(q, k)
+    with pytest.raises(ValueError):
+        ops.attn_bwd(q, k, v, o, lse, do, causal=True, workspace=small, keep_ds=True)
