@@ -291,7 +291,10 @@ def main():
     f_fwd, f_bwd = attn_flops(L, L, H, D)
     # algorithmic FLOPs per launch: the backward's 5 tile products are S, dP, dV, dK (in the
     # dK/dV kernel) and dQ (in the dQ kernel); the S and dP the dQ kernel recomputes are not counted
-    algo = {"attn_fwd_w8": f_fwd, "attn_bwd_dkdv_pipe": f_bwd * 4 / 5, "attn_bwd_dq_pipe": f_bwd * 1 / 5}
+    # (with kept dS -- ops.attn_bwd's default where the scratch fits -- the dQ kernel is the one product, over
+    # the dS tiles that the dK/dV kernel stored: 2 bytes per visible pair each way)
+    dq_kernel = "attn_bwd_dq_kept" if "attn_bwd_dq_kept" in prof else "attn_bwd_dq_pipe"
+    algo = {"attn_fwd_w8": f_fwd, "attn_bwd_dkdv_pipe": f_bwd * 4 / 5, dq_kernel: f_bwd * 1 / 5}
     missing = [n for n in algo if n not in prof]
     if missing:
         raise SystemExit(f"bench.py: the library ran no kernel named {missing}; it reported {sorted(prof)}")
@@ -301,6 +304,10 @@ def main():
         kernels[name] = {"launches": n, "avg_ms": round(avg, 4), "min_ms": round(min_ms, 4)}
         if name in algo:
             kernels[name]["tflops"] = round(algo[name] / (avg * 1e-3) / 1e12, 1)
+        if name == "attn_bwd_dq_kept":   # bound by HBM: the kept dS, read once
+            ds_bytes = _lib.load().ody_attn_bwd_ds_bytes(1, L, L, H, HKV, D, _lib.ODY_BF16, 1)
+            kernels[name]["hbm_read_gbps"] = round(ds_bytes / (avg * 1e-3) / 1e9, 1)
+            kernels[name]["frac_of_hbm_peak"] = round(ds_bytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 3)
     dom = max(algo, key=lambda n: prof[n][1] / prof[n][0])
     dom_avg = prof[dom][1] / prof[dom][0]
     achieved = algo[dom] / (dom_avg * 1e-3) / 1e12

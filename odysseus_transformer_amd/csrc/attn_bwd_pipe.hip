@@ -283,7 +283,8 @@ constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q,
 // contiguous, key block after key block, and inside a key block by qb.  Entries of masked pairs are 0; the parts
 // (y, x) of a diagonal block with y > x, whose keys all come after their queries, are never written (and never used).
 constexpr int DS_PIECE = 64 * 8;                 // one (y, x, c): 1 KB
-constexpr int DS_BLOCK_ELEMS = 4 * 4 * 8 * DS_PIECE;
+constexpr int DS_PART = 4 * 8 * DS_PIECE;        // one y: 32 KB
+constexpr int DS_BLOCK_ELEMS = 4 * DS_PART;
 __host__ __device__ inline int64_t ds_blocks_per_head(int nb) { return (int64_t)nb * (nb + 1) / 2; }
 __host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
   return (int64_t)kb * nb - (int64_t)kb * (kb - 1) / 2 + (qb - kb);
@@ -301,7 +302,7 @@ __host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
 // kv heads this is what gives the chip enough, and evenly sized, blocks.
 //
 // KEEP_DS = true (causal self-attention, Lq == Lk a multiple of 256): every dS tile also goes to p.ds, in the
-// layout described at ds_block_index, and the dQ kernel below (attn_bwd_dq_from_ds_kernel) reads it back
+// layout described at ds_block_index, and the dQ kernel below (attn_bwd_dq_kept_kernel) reads it back
 // instead of computing S, dP and dS a second time.
 template <bool SPLIT, bool KEEP_DS>
 __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const AttnParams p,
@@ -548,21 +549,33 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 // ---------------------------------------------------------------------------------
 // One product, dQ^T += K^T dS^T, over the tiles that the dK/dV kernel (KEEP_DS) left in p.ds.  256 queries per block,
 // 8 wavefronts x 32 queries: wavefront w owns chunks 4 (w & 1) ... + 3 of 64-query tile (w >> 1) of the block, lane i
-// the query at position 32 (w & 1) + i of that tile's kept order.  A three-deep ring of {the 32 one-KB pieces of dS
-// that belong to this 64-key tile and the block's 4 query tiles, K^T image}.
+// the query at position 32 (w & 1) + i of that tile's kept order.
 //
-//      A: K^T image (LDS, 16-byte reads), as in the dQ kernel above
+//      A: K^T image (LDS, 16-byte reads), as in the dQ kernel at the top of this file
 //      B: dS^T.  The tiles hold 8 queries of one key side by side, the product contracts over keys: the transposing
 //         LDS read turns 4 keys x 16 queries into 4-key pieces per query, two of them make a fragment.
 //
-// 2 bytes per visible (query, key) pair for 256 flops: the kernel is bound by HBM, half of the matrix pipe idles.
+// 2 bytes per visible (query, key) pair for 256 flops: the kernel is bound by HBM, and what it needs is bytes in
+// flight -- more than the LDS could take as landing room.  So the dS of a 64-key tile (32 one-KB pieces, 4 per
+// wavefront) and its K^T image (2 KB per wavefront) travel through registers: four sets, loaded four tiles ahead,
+// written to one of two LDS buffers the iteration before their tile is due.  (Direct loads to LDS for the images
+// would put two kinds of loads on the one counter, and the compiler then waits for all of them every time.)
+// The compiler places the waits for the register loads by counting the loads issued since, so these must leave in
+// program order: no pass may move a load across this point, neither the optimizer nor the instruction scheduler.
+#define ISSUE_ORDER()                    \
+  do {                                   \
+    asm volatile("" ::: "memory");       \
+    __builtin_amdgcn_sched_barrier(0);   \
+  } while (0)
 constexpr int DS_PIECE_ELEMS = GROUP_ELEMS;   // 1 KB + 16 bytes: consecutive pieces start 4 banks apart
-constexpr int DQS_STAGE = 32 * DS_PIECE_ELEMS + IMG_ELEMS;
+constexpr int DQK_DS_BUF = 32 * DS_PIECE_ELEMS, DQK_SETS = 4;
+constexpr int DQK_LDS_ELEMS = 2 * DQK_DS_BUF + 2 * IMG_ELEMS;
 
-__global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_from_ds_kernel(const AttnParams p,
-                                                                          const bf16* __restrict__ kimg) {
+__global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const AttnParams p, const bf16* __restrict__ kimg) {
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  bf16* ring = reinterpret_cast<bf16*>(smem_raw);     // [3][DQS_STAGE]
+  bf16* dsbuf = reinterpret_cast<bf16*>(smem_raw);   // [2][DQK_DS_BUF]
+  bf16* imgs = dsbuf + 2 * DQK_DS_BUF;               // [2][IMG_ELEMS]
 
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
             i = lane & 31;
@@ -570,29 +583,39 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_from_ds_kernel(const A
   const int nqb = gridDim.x / (p.Hq * p.B);
   const int qblk = nqb - 1 - bc.rank;   // heaviest blocks first
   const int h = bc.h, b = bc.b, hk = h / p.group;
-  const int q_tiles = p.Lq / KV_BQ, x = wave >> 1, mt = wave & 1;
+  const int q_tiles = p.Lq / KV_BQ, x = wave >> 1, mt = wave & 1, nb = q_tiles / 4;
   const bf16* kip = kimg + ((int64_t)b * p.Hkv + hk) * (p.Lk / 64) * IMG_ELEMS;
-  const int nb = q_tiles / 4;
   const bf16* dsh = p.ds + ((int64_t)b * p.Hq + h) * ds_blocks_per_head(nb) * DS_BLOCK_ELEMS;
-  const int ntiles = 4 * (qblk + 1);   // 64-key tiles up to the block's last query
+  const int ntiles = 4 * (qblk + 1);   // 64-key tiles up to the block's last query; a multiple of DQK_SETS
 
-  auto load_part = [&](bf16* st, int t, int j) {   // j = 0, 1: the two halves of a stage's loads
-    // the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk): 32 KB in a row
-    const bf16* src = dsh + ds_block_index(nb, t >> 2, qblk) * DS_BLOCK_ELEMS + (t & 3) * (32 * DS_PIECE);
+  u32x4 regs[DQK_SETS][6];
+  // tile t: this wavefront's 4 of the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk) -- 32 KB in a row --
+  // and its 2 of the 16 KB of the K^T image, into register set `set`
+  auto issue = [&](int set, int t) {
+    const bf16* src = dsh + ds_block_index(nb, t >> 2, qblk) * DS_BLOCK_ELEMS + (t & 3) * DS_PART;
 #pragma unroll
-    for (int n = 0; n < 2; n++) {
-      const int piece = 8 * (2 * j + n) + wave;   // query tile 2 j + n of the block, chunk `wave`
-      __builtin_amdgcn_global_load_lds((global_void_ptr)(src + (unsigned)(piece * DS_PIECE + lane * 8)),
-                                       (lds_void_ptr)(st + piece * DS_PIECE_ELEMS), 16, 0, 0);
+    for (int n = 0; n < 4; n++) {   // piece 8 n + wave: query tile n of the block, chunk `wave`
+      regs[set][n] = *reinterpret_cast<const u32x4*>(src + (unsigned)((8 * n + wave) * DS_PIECE + lane * 8));
+      ISSUE_ORDER();
     }
-    const int grp = DQ_WAVES * j + wave;
-    __builtin_amdgcn_global_load_lds((global_void_ptr)(kip + (int64_t)t * IMG_ELEMS + (grp * 64 + lane) * 8),
-                                     (lds_void_ptr)(st + 32 * DS_PIECE_ELEMS + grp * 512), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      regs[set][4 + j] = *reinterpret_cast<const u32x4*>(kip + (int64_t)t * IMG_ELEMS + (unsigned)(((DQ_WAVES * j + wave) * 64 + lane) * 8));
+      ISSUE_ORDER();
+    }
   };
-  load_part(ring, 0, 0);
-  load_part(ring, 0, 1);
-  load_part(ring + DQS_STAGE, 1, 0);   // ntiles >= 4
-  load_part(ring + DQS_STAGE, 1, 1);
+  auto drain = [&](int set, int t) {
+    bf16* buf = dsbuf + (t & 1) * DQK_DS_BUF;
+#pragma unroll
+    for (int n = 0; n < 4; n++)
+      *reinterpret_cast<u32x4*>(buf + (8 * n + wave) * DS_PIECE_ELEMS + lane * 8) = regs[set][n];
+    bf16* slot = imgs + (t & 1) * IMG_ELEMS;
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+      *reinterpret_cast<u32x4*>(slot + ((DQ_WAVES * j + wave) * 64 + lane) * 8) = regs[set][4 + j];
+  };
+#pragma unroll
+  for (int u = 0; u < DQK_SETS; u++) issue(u, u);   // ntiles >= DQK_SETS
 
   f32x16 dq[DT];
 #pragma unroll
@@ -606,9 +629,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_from_ds_kernel(const A
   const int sbase = (8 * x + 4 * mt + 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1)) * DS_PIECE_ELEMS +
                     (16 * g + 4 * ((lane >> 2) & 3)) * 8 + 4 * (lane & 1);
 
-  auto tile = [&](const bf16* st) {
-    const bf16* Sp = st + sbase;
-    const bf16* Ki = st + 32 * DS_PIECE_ELEMS;
+  auto tile = [&](int t) {
+    const bf16* Sp = dsbuf + (t & 1) * DQK_DS_BUF + sbase;
+    const bf16* Ki = imgs + (t & 1) * IMG_ELEMS;
     constexpr int IPF = 4;
     bf16x8 ifr[IPF], dsf[2][2];
 #pragma unroll
@@ -631,19 +654,27 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_from_ds_kernel(const A
     }
   };
 
-  for (int t = 0; t < ntiles; t++) {
-    // stage t landed (the loads of stage t+1 may still be in flight), everyone done with stage t-1
-    if (t + 1 < ntiles) {
-      asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    // the loads go first: what bounds this kernel is the time a tile spends on its way from HBM, and issued here
-    // a tile has two iterations to arrive
-    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * DQS_STAGE, t + 2, 0);
-    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * DQS_STAGE, t + 2, 1);
-    // tiles whose keys all come after this wavefront's queries were never written
-    if (t <= 4 * qblk + x) tile(ring + (t % 3) * DQS_STAGE);
-  }
+  drain(0, 0);
+  ISSUE_ORDER();
+  int t0 = 0;
+  do {   // not a `for`: its entry test would give the compiler a block to sink the loads above into, out of order
+#pragma unroll
+    for (int u = 0; u < DQK_SETS; u++) {
+      const int t = t0 + u;
+      // everyone is done with tile t - 1, and sees what the wavefronts wrote of tile t to LDS an iteration ago
+      __syncthreads();
+      // tile t + 1 has arrived (the compiler places the wait: all loads are of one kind, so it can count them);
+      // tiles t + 2 and t + 3 may still be on their way, and tile t + 4 sets out
+      // No branches around these (past the end: a write that nobody reads, and one more load of the last tile):
+      // with branches the compiler loses count of the loads in flight and waits for all of them.
+      ISSUE_ORDER();
+      drain((u + 1) % DQK_SETS, t + 1);
+      ISSUE_ORDER();
+      issue(u, min(t + DQK_SETS, ntiles - 1));
+      // tiles whose keys all come after this wavefront's queries were never written
+      if (t <= 4 * qblk + x) tile(t);
+    }
+  } while ((t0 += DQK_SETS) < ntiles);
 
   // position 32 mt + i of the tile's kept order = chunk 4 mt + (i >> 3), element i & 7
   const int row = 32 * ((i >> 2) & 1) + 16 * ((i >> 3) & 1) + 4 * (i & 3) + (i >> 4) + 2 * mt;
@@ -717,10 +748,10 @@ size_t ody_attn_bwd_pipe_ds_bytes(int B, int Lq, int Lk, int Hq, int causal) {
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
   constexpr size_t smem_q = (size_t)3 * (2 * TILE_ELEMS + IMG_ELEMS) * sizeof(bf16);
   constexpr size_t smem_kv = (size_t)2 * KV_STAGE * sizeof(bf16);
-  constexpr size_t smem_qs = (size_t)3 * DQS_STAGE * sizeof(bf16);
+  constexpr size_t smem_qs = (size_t)DQK_LDS_ELEMS * sizeof(bf16);
   static_assert(smem_qs <= 160 * 1024, "LDS of one CU");
   for (const auto& ks : {std::pair<const void*, size_t>{reinterpret_cast<const void*>(&attn_bwd_dq_pipe_kernel), smem_q},
-                         {reinterpret_cast<const void*>(&attn_bwd_dq_from_ds_kernel), smem_qs},
+                         {reinterpret_cast<const void*>(&attn_bwd_dq_kept_kernel), smem_qs},
                          {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false, false>), smem_kv},
                          {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<true, false>), smem_kv},
                          {reinterpret_cast<const void*>(&attn_bwd_dkdv_pipe_kernel<false, true>), smem_kv},
@@ -767,8 +798,8 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
     // what ody_attn_bwd_pipe_ds_bytes promised: whole 256-row blocks on both sides, queries and keys aligned
     ODY_REQUIRE(p.causal && p.off == 0 && p.Lq % KV_BN == 0 && KV_BN == DQ_BM, ODY_ERR_UNSUPPORTED,
                 "attn_bwd: kept dS needs causal self-attention on a multiple of %d rows", KV_BN);
-    ODY_LAUNCH("attn_bwd_dq_from_ds", st, attn_bwd_dq_from_ds_kernel, gq, dim3(DQ_THREADS), smem_qs, p, kimg);
-    return ody_check_launch("attn_bwd_dq_from_ds");
+    ODY_LAUNCH("attn_bwd_dq_kept", st, attn_bwd_dq_kept_kernel, gq, dim3(DQ_THREADS), smem_qs, p, kimg);
+    return ody_check_launch("attn_bwd_dq_kept");
   }
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");

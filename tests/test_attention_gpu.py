@@ -267,11 +267,11 @@ def test_attention_bwd_kept_ds_policy(dev):
         finally:
             _lib.profile_enable(False)
 
-    assert "attn_bwd_dq_from_ds" in kernels()
+    assert "attn_bwd_dq_kept" in kernels()
     ops.set_keep_ds_max_bytes(0)
     try:
         assert "attn_bwd_dq_pipe" in kernels()
-        assert "attn_bwd_dq_from_ds" in kernels(keep_ds=True)
+        assert "attn_bwd_dq_kept" in kernels(keep_ds=True)
     finally:
         ops.set_keep_ds_max_bytes(None)
     with pytest.raises(ValueError):
