@@ -268,11 +268,11 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
 // ring as row tiles (A operands of S and dP) and as transposed images (A operands of dV^T and
 // dK^T); P and dS are accumulator tiles, which is the B-operand layout of the next product.
 //
-//      S  = Q K^T - lse/scale     -lse/scale enters as one more k-step of the contraction, so P = exp2(S c)
+//      S  = Q K^T - lse/scale     the accumulators start at -lse/scale, so P = exp2(S c)
 //      dP = dO V^T - delta        likewise -delta
 //      dV^T += dO^T P             dK^T += Q^T (P o dP)
 constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 * KV_WAVES;
-constexpr int KV_STAT_ELEMS = 128 * 8;                                   // start-value fragments of one tile
+constexpr int KV_STAT_ELEMS = 64 * 8;                                    // start-value record of one tile: 1 KB, one direct load
 constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q, dO tiles; Q^T, dO^T images; start values
 
 // dS kept for the dQ kernel (causal, Lq == Lk, a multiple of 256): one 128 KB block per (256-key block kb, 256-query
@@ -290,11 +290,13 @@ __host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
   return (int64_t)kb * nb - (int64_t)kb * (kb - 1) / 2 + (qb - kb);
 }
 
-// The start values of S and dP for every 64-query tile enter as one more A-operand fragment of the contraction
-// (the matching B fragment is all ones): the fp32 value x is split into three bf16 terms x = h + m + l, which
-// the MFMA adds up exactly like any other product.  The query-side pre-pass (attn_bwd_prepass_kernel) writes
-// them: per (batch, head, tile) [sub-tile mt][0: -lse/scale, 1: -delta][MFMA row i][8 bf16], row i of sub-tile
-// mt being query tile_row(i, mt).  Rows that must give P = 0 (beyond Lq, or a query that saw no key) hold -1e30.
+// S and dP do not start from zero: the accumulators of a sub-tile are loaded with -lse/scale and -delta of their
+// rows, so that S comes out of the MFMAs as q.k - lse/scale and P = exp2(S c) costs one multiply and one exp per
+// element.  A lane's 16 accumulator rows depend on its lane group only, so the 32 lanes of a group read the same 16
+// floats (4 broadcast reads of 16 bytes per product).  The query-side pre-pass (attn_bwd_prepass_kernel) writes them:
+// per (batch, head, tile) a table [sub-tile mt][0: -lse/scale, 1: -delta][lane group g][register r] of fp32 at the
+// start of a 1 KB record, register r of group g being query acc_tile_row(r, g, mt).  Rows that must give P = 0
+// (beyond Lq, or a query that saw no key) hold -1e30.
 //
 // SPLIT = false: a block owns 256 keys of one kv head and walks all query heads of its group.
 // SPLIT = true (grouped-query attention): a block owns 256 keys for ONE query head and writes
@@ -359,10 +361,9 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     const bf16* doi = doimg + tile_id * IMG_ELEMS;
     const int rmax = p.Lq - 1 - t * KV_BQ;   // rows beyond the matrix re-read its last row
     const int ln = fresh_lane();
-    if (j == 0 && wave >= KV_WAVES - 2)
-      __builtin_amdgcn_global_load_lds(
-          (global_void_ptr)(stats + tile_id * KV_STAT_ELEMS + (unsigned)(((wave - (KV_WAVES - 2)) * 64 + ln) * 8)),
-          (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS + (wave - (KV_WAVES - 2)) * 512), 16, 0, 0);
+    if (j == 0 && wave == KV_WAVES - 1)
+      __builtin_amdgcn_global_load_lds((global_void_ptr)(stats + tile_id * KV_STAT_ELEMS + (unsigned)(ln * 8)),
+                                       (lds_void_ptr)(st + 2 * TILE_ELEMS + 2 * IMG_ELEMS), 16, 0, 0);
     {
       const int grp = KV_WAVES * j + wave;
       const int row = min(4 * grp + (ln >> 4), rmax), col = 8 * (ln & 15);
@@ -381,8 +382,8 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     load_stage(ring, 0, 1);
   }
 
-  // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP, the vector
-  // work, 16 MFMAs for dV^T and dK^T
+  // one 32-query sub-tile against this wavefront's 32 keys: 16 MFMAs for S and dP on top of their
+  // start values, the vector work, 16 MFMAs for dV^T and dK^T
   // kept dS: chunk 4 mt + 2 ss + g of part (y, x) = (wave >> 1, t & 3) of the block, to which `tile` points at this
   // wavefront's 32 keys.  Streaming stores: the tiles are read once, by another kernel.
   auto sub_tile = [&](const bf16* st, int t, int mt, bool masked, bf16* ds_tile) {
@@ -392,17 +393,20 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     const bf16* Ot = st + TILE_ELEMS;
     const bf16* Qi = st + 2 * TILE_ELEMS;
     const bf16* Oi = Qi + IMG_ELEMS;
-    const bf16* St = Oi + IMG_ELEMS + mt * 512 + i * 8;
     constexpr int PF = 2;
     bf16x8 qfr[PF], ofr[PF];
-    const bf16x8 s0 = *reinterpret_cast<const bf16x8*>(St), d0 = *reinterpret_cast<const bf16x8*>(St + 256);
+    f32x16 s, dp;
+    {
+      const float* Sf = reinterpret_cast<const float*>(Oi + IMG_ELEMS) + mt * 64 + g * 16;
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(Sf + 4 * a), w = *reinterpret_cast<const f32x4*>(Sf + 32 + 4 * a);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s[4 * a + e] = v[e], dp[4 * a + e] = w[e];
+      }
+    }
     qfr[0] = row_frag(Qt, rbase, 0, mt);
     ofr[0] = row_frag(Ot, rbase, 0, mt);
-    const bf16 one = (bf16)(g == 0 ? 1.f : 0.f), zero = (bf16)0.f;
-    const bf16x8 ones = {one, one, one, zero, zero, zero, zero, zero};   // k-slots 0..2 carry the start value
-    FENCE();
-    f32x16 s = mfma32(s0, ones, f32x16{0});
-    f32x16 dp = mfma32(d0, ones, f32x16{0});
     qfr[1] = row_frag(Qt, rbase, 1, mt);
     ofr[1] = row_frag(Ot, rbase, 1, mt);
     FENCE();

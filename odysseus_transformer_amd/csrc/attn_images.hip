@@ -43,9 +43,9 @@ __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict
 }
 
 // The whole query side of the head_dim-128 backward in one pass over Q, dO and O (one block per 64-query tile of a
-// head): delta = sum_d dO * O, the transposed images of the Q tile and of the dO tile, and the tile's start-value
-// fragments (-lse / scale and -delta, each split into three bf16 terms; layout described where the dK/dV kernel reads
-// them).  Replaces four launches that each went over the same rows.
+// head): delta = sum_d dO * O, the transposed images of the Q tile and of the dO tile, and the tile's start values
+// (-lse / scale and -delta in the order of the dK/dV kernel's accumulator registers; layout described where that
+// kernel reads them).  Replaces four launches that each went over the same rows.
 __global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams p, bf16* __restrict__ qimg,
                                                                bf16* __restrict__ doimg, bf16* __restrict__ stats) {
   constexpr int PITCH = 128 + 8;
@@ -100,8 +100,9 @@ __global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams 
     }
   }
   if (tid < 128) {
-    const int mt = tid >> 6, which = (tid >> 5) & 1, i = tid & 31;
-    const int row = tile_row(i, mt), qi = t * 64 + row;
+    // fp32 table [sub-tile mt][0: -lse/scale, 1: -delta][lane group g][accumulator register r]
+    const int mt = tid >> 6, which = (tid >> 5) & 1, g = (tid >> 4) & 1, r = tid & 15;
+    const int row = acc_tile_row(r, g, mt), qi = t * 64 + row;
     float x;
     if (which == 0) {
       const float l = (qi < p.Lq) ? p.lse[((int64_t)b * p.Hq + h) * p.Lq + qi] : INFINITY;
@@ -109,11 +110,7 @@ __global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams 
     } else {
       x = (qi < p.Lq) ? -sdelta[row] : 0.f;
     }
-    const bf16 hi = (bf16)x;
-    const bf16 mid = (bf16)(x - (float)hi);
-    const bf16 lo = (bf16)(x - (float)hi - (float)mid);
-    const bf16 z = (bf16)0.f;
-    *reinterpret_cast<bf16x8*>(stats + (tile_id * 128 + tid) * 8) = bf16x8{hi, mid, lo, z, z, z, z, z};
+    reinterpret_cast<float*>(stats)[tile_id * 256 + tid] = x;   // records of 1 KB
   }
 }
 

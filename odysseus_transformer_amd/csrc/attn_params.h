@@ -59,7 +59,7 @@ size_t ody_attn_images_bytes(int B, int L, int H);
 int ody_launch_attn_images(const void* src, const AttnStrides& s, int B, int L, int H, void* dst, int* flags,
                            int nflags, hipStream_t st);
 // head_dim 128 backward, everything that depends on the queries only, in one launch: p.delta, the transposed images
-// of Q and dO and the start-value fragments of every 64-query tile
+// of Q and dO and the start values (1 KB per 64-query tile)
 int ody_launch_attn_bwd_prepass(const AttnParams& p, void* qimg, void* doimg, void* stats, hipStream_t st);
 // head_dim 128 only, 8 wavefronts x 32 queries per block; workspace of ody_attn_fwd_w8_workspace(...) bytes
 int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, hipStream_t st);
