@@ -146,10 +146,11 @@ int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out,
  *   ODY_BWD_KEEP_DS           spends memory to save arithmetic (no counterpart in the reference): the dK/dV
  *                             kernel keeps dS, rounded to bf16 as it is used there, in the workspace, and dQ is
  *                             one product dS K over it instead of a second pass over S, dP and dS.  Same
- *                             results.  For bf16, head_dim 128, causal, Lq == Lk a multiple of 256
- *                             (ody_attn_bwd_ds_bytes(...) > 0); the workspace then holds
+ *                             results.  For bf16, head_dim 128, Lq and Lk multiples of 256 and, if causal,
+ *                             Lq == Lk (ody_attn_bwd_ds_bytes(...) > 0); the workspace then holds
  *                             ody_attn_bwd_workspace_bytes(...) + ody_attn_bwd_ds_bytes(...) bytes, the latter
- *                             about B * Hq * Lq * Lq bytes (2 bytes per visible pair).
+ *                             2 bytes per visible (query, key) pair: about B * Hq * Lq * Lk bytes when causal,
+ *                             twice that for a full block.
  * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
  * the bf16 head_dim-128 kernels transposed copies of K, Q and dO).
  */

@@ -186,7 +186,7 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
   if (flags & ODY_BWD_KEEP_DS) {
     ws_ds = ody_attn_bwd_ds_bytes(B, Lq, Lk, Hq, Hkv, D, dtype, causal);
     ODY_REQUIRE(ws_ds > 0, ODY_ERR_UNSUPPORTED,
-                "%s: ODY_BWD_KEEP_DS needs bf16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256", who);
+                "%s: ODY_BWD_KEEP_DS needs bf16, head_dim 128, Lq and Lk multiples of 256 and, if causal, Lq == Lk", who);
   }
   ODY_REQUIRE(workspace_bytes >= ws_base + ws_ds, ODY_ERR_WORKSPACE, "%s: workspace of %zu bytes, %zu needed", who,
               workspace_bytes, ws_base + ws_ds);

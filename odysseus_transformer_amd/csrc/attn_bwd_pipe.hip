@@ -275,8 +275,8 @@ constexpr int KV_WAVES = 8, KV_BN = 32 * KV_WAVES, KV_BQ = 64, KV_THREADS = 64 *
 constexpr int KV_STAT_ELEMS = 64 * 8;                                    // start-value record of one tile: 1 KB, one direct load
 constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q, dO tiles; Q^T, dO^T images; start values
 
-// dS kept for the dQ kernel (causal, Lq == Lk, a multiple of 256): one 128 KB block per (256-key block kb, 256-query
-// block qb >= kb), laid out for the reader, which takes 64 keys x 256 queries at a time:
+// dS kept for the dQ kernel (Lq and Lk multiples of 256; causal: Lq == Lk): one 128 KB block per (256-key block kb,
+// 256-query block qb; causal: qb >= kb), laid out for the reader, which takes 64 keys x 256 queries at a time:
 //   [64-key tile y = 0..3][64-query tile x = 0..3][chunk c = 0..7][key 0..63][8 bf16]
 // Element j of chunk c is the query of tile row 32 (j >> 2) + 16 (c & 1) + 4 (j & 3) + ((c >> 1) & 1) + 2 (c >> 2) -- the
 // order in which an accumulator holds the rows, i.e. image_pos(row) = 8 c + j.  Blocks of one (batch, head) are
@@ -285,9 +285,12 @@ constexpr int KV_STAGE = 2 * TILE_ELEMS + 2 * IMG_ELEMS + KV_STAT_ELEMS;   // Q,
 constexpr int DS_PIECE = 64 * 8;                 // one (y, x, c): 1 KB
 constexpr int DS_PART = 4 * 8 * DS_PIECE;        // one y: 32 KB
 constexpr int DS_BLOCK_ELEMS = 4 * DS_PART;
-__host__ __device__ inline int64_t ds_blocks_per_head(int nb) { return (int64_t)nb * (nb + 1) / 2; }
-__host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
-  return (int64_t)kb * nb - (int64_t)kb * (kb - 1) / 2 + (qb - kb);
+// nbq, nbk: 256-row blocks of queries and of keys.  Causal (nbq == nbk): the blocks at or below the diagonal.
+__host__ __device__ inline int64_t ds_blocks_per_head(int nbq, int nbk, bool causal) {
+  return causal ? (int64_t)nbq * (nbq + 1) / 2 : (int64_t)nbq * nbk;
+}
+__host__ __device__ inline int64_t ds_block_index(int nbq, int kb, int qb, bool causal) {
+  return causal ? (int64_t)kb * nbq - (int64_t)kb * (kb - 1) / 2 + (qb - kb) : (int64_t)kb * nbq + qb;
 }
 
 // S and dP do not start from zero: the accumulators of a sub-tile are loaded with -lse/scale and -delta of their
@@ -303,7 +306,7 @@ __host__ __device__ inline int64_t ds_block_index(int nb, int kb, int qb) {
 // fp32 partial dK / dV to `part`, which attn_bwd_group_sum_kernel adds up over the group.  With few
 // kv heads this is what gives the chip enough, and evenly sized, blocks.
 //
-// KEEP_DS = true (causal self-attention, Lq == Lk a multiple of 256): every dS tile also goes to p.ds, in the
+// KEEP_DS = true (whole 256-row blocks on both sides; causal: self-attention): every dS tile also goes to p.ds, in the
 // layout described at ds_block_index, and the dQ kernel below (attn_bwd_dq_kept_kernel) reads it back
 // instead of computing S, dP and dS a second time.
 template <bool SPLIT, bool KEEP_DS>
@@ -475,8 +478,9 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     const bool masked = p.causal && (t * KV_BQ + p.off < wn0 + 31);
     bf16* ds_tile = nullptr;
     if (KEEP_DS) {
-      const int nb = q_tiles / 4;
-      ds_tile = p.ds + (((int64_t)b * p.Hq + h_first + it / ntq) * ds_blocks_per_head(nb) + ds_block_index(nb, bc.rank, t >> 2)) * DS_BLOCK_ELEMS +
+      const int nbq = q_tiles / 4, nbk = p.Lk / KV_BN;
+      ds_tile = p.ds + (((int64_t)b * p.Hq + h_first + it / ntq) * ds_blocks_per_head(nbq, nbk, p.causal) +
+                        ds_block_index(nbq, bc.rank, t >> 2, p.causal)) * DS_BLOCK_ELEMS +
                 (((wave >> 1) * 4 + (t & 3)) * 8) * DS_PIECE + (wave & 1) * 32 * 8;
     }
 #pragma unroll 1
@@ -585,18 +589,20 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
             i = lane & 31;
   const BlockCoord bc = ody_block_coord(p.Hq, p.B);
   const int nqb = gridDim.x / (p.Hq * p.B);
-  const int qblk = nqb - 1 - bc.rank;   // heaviest blocks first
+  const int qblk = p.causal ? nqb - 1 - bc.rank : bc.rank;   // causal: heaviest blocks first
   const int h = bc.h, b = bc.b, hk = h / p.group;
-  const int q_tiles = p.Lq / KV_BQ, x = wave >> 1, mt = wave & 1, nb = q_tiles / 4;
+  const int x = wave >> 1, mt = wave & 1, nbq = p.Lq / KV_BN, nbk = p.Lk / KV_BN;
   const bf16* kip = kimg + ((int64_t)b * p.Hkv + hk) * (p.Lk / 64) * IMG_ELEMS;
-  const bf16* dsh = p.ds + ((int64_t)b * p.Hq + h) * ds_blocks_per_head(nb) * DS_BLOCK_ELEMS;
-  const int ntiles = 4 * (qblk + 1);   // 64-key tiles up to the block's last query; a multiple of DQK_SETS
+  const bf16* dsh = p.ds + ((int64_t)b * p.Hq + h) * ds_blocks_per_head(nbq, nbk, p.causal) * DS_BLOCK_ELEMS;
+  // 64-key tiles: all of them, or (causal) those up to the block's last query; a multiple of DQK_SETS
+  const int ntiles = p.causal ? 4 * (qblk + 1) : 4 * nbk;
+  const int last_tile = p.causal ? 4 * qblk + x : ntiles;   // of this wavefront's queries
 
   u32x4 regs[DQK_SETS][6];
   // tile t: this wavefront's 4 of the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk) -- 32 KB in a row --
   // and its 2 of the 16 KB of the K^T image, into register set `set`
   auto issue = [&](int set, int t) {
-    const bf16* src = dsh + ds_block_index(nb, t >> 2, qblk) * DS_BLOCK_ELEMS + (t & 3) * DS_PART;
+    const bf16* src = dsh + ds_block_index(nbq, t >> 2, qblk, p.causal) * DS_BLOCK_ELEMS + (t & 3) * DS_PART;
 #pragma unroll
     for (int n = 0; n < 4; n++) {   // piece 8 n + wave: query tile n of the block, chunk `wave`
       regs[set][n] = *reinterpret_cast<const u32x4*>(src + (unsigned)((8 * n + wave) * DS_PIECE + lane * 8));
@@ -675,8 +681,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
       drain((u + 1) % DQK_SETS, t + 1);
       ISSUE_ORDER();
       issue(u, min(t + DQK_SETS, ntiles - 1));
-      // tiles whose keys all come after this wavefront's queries were never written
-      if (t <= 4 * qblk + x) tile(t);
+      // (causal) tiles whose keys all come after this wavefront's queries were never written
+      if (t <= last_tile) tile(t);
     }
   } while ((t0 += DQK_SETS) < ntiles);
 
@@ -745,8 +751,8 @@ size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
 }
 
 size_t ody_attn_bwd_pipe_ds_bytes(int B, int Lq, int Lk, int Hq, int causal) {
-  if (!causal || Lq != Lk || Lq % KV_BN != 0 || B <= 0 || Hq <= 0) return 0;
-  return (size_t)B * Hq * ds_blocks_per_head(Lq / KV_BN) * DS_BLOCK_ELEMS * sizeof(bf16);
+  if (Lq % KV_BN != 0 || Lk % KV_BN != 0 || (causal && Lq != Lk) || B <= 0 || Hq <= 0) return 0;
+  return (size_t)B * Hq * ds_blocks_per_head(Lq / KV_BN, Lk / KV_BN, causal != 0) * DS_BLOCK_ELEMS * sizeof(bf16);
 }
 
 int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t st) {
@@ -800,8 +806,8 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
   if (p.ds) {
     // what ody_attn_bwd_pipe_ds_bytes promised: whole 256-row blocks on both sides, queries and keys aligned
-    ODY_REQUIRE(p.causal && p.off == 0 && p.Lq % KV_BN == 0 && KV_BN == DQ_BM, ODY_ERR_UNSUPPORTED,
-                "attn_bwd: kept dS needs causal self-attention on a multiple of %d rows", KV_BN);
+    ODY_REQUIRE(p.Lq % KV_BN == 0 && p.Lk % KV_BN == 0 && (!p.causal || p.off == 0) && KV_BN == DQ_BM, ODY_ERR_UNSUPPORTED,
+                "attn_bwd: kept dS needs multiples of %d rows on both sides and, if causal, as many keys as queries", KV_BN);
     ODY_LAUNCH("attn_bwd_dq_kept", st, attn_bwd_dq_kept_kernel, gq, dim3(DQ_THREADS), smem_qs, p, kimg);
     return ody_check_launch("attn_bwd_dq_kept");
   }

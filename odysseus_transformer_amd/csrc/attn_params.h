@@ -28,7 +28,7 @@ struct AttnParams {
   // gradient of the projection BEFORE its rotary embedding
   const bf16* rope_q;
   const bf16* rope_k;
-  // bwd, bf16 head_dim 128, causal self-attention with Lq == Lk a multiple of 256: when set, the dK/dV kernel keeps
+  // bwd, bf16 head_dim 128, Lq and Lk multiples of 256 (causal: Lq == Lk): when set, the dK/dV kernel keeps
   // every dS tile here (ody_attn_bwd_ds_bytes) and dQ is computed from them instead of from a second pass over S and dP
   bf16* ds;
   float scale;        // softmax scale

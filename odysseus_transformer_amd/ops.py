@@ -122,8 +122,8 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     head_dim 128) makes dq and dk the gradients of the projection BEFORE its rotary embedding.
 
     keep_ds spends scratch memory to save arithmetic: the dK/dV kernel keeps dS (2 bytes per visible
-    query-key pair, about B * Hq * L * L bytes) and dQ becomes one product over it instead of a second
-    pass over S and dP.  bfloat16, head_dim 128, causal, Lq == Lk a multiple of 256 only.  None (the
+    query-key pair: about B * Hq * L * L bytes when causal) and dQ becomes one product over it instead of a second
+    pass over S and dP.  bfloat16, head_dim 128, Lq and Lk multiples of 256, causal only with Lq == Lk.  None (the
     default) turns it on where the shape qualifies, no `workspace` is passed and the scratch stays within
     keep_ds_max_bytes(); True insists (ValueError where the shape does not qualify); False never."""
     _need_gpu(q, k, v, out, lse, dout)
@@ -147,7 +147,7 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     ws_bytes = lib.ody_attn_bwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
     ds_bytes = lib.ody_attn_bwd_ds_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q), int(causal)) if keep_ds is not False else 0
     if keep_ds and ds_bytes == 0:
-        raise ValueError("keep_ds needs bfloat16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256")
+        raise ValueError(_KEEP_DS_SHAPES)
     ws = None
     if keep_ds is None:
         keep_ds = workspace is None and 0 < ds_bytes <= keep_ds_max_bytes(q.device)
@@ -189,6 +189,7 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
 
 
 _KEEP_DS_MAX_BYTES: Optional[int] = None
+_KEEP_DS_SHAPES = "keep_ds needs bfloat16, head_dim 128, Lq and Lk multiples of 256 and, if causal, Lq == Lk"
 
 
 def keep_ds_max_bytes(device=None) -> int:
@@ -217,9 +218,41 @@ def attn_bwd_workspace(q, k, keep_ds: bool = False, causal: bool = True) -> torc
     if keep_ds:
         ds = lib.ody_attn_bwd_ds_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q), int(causal))
         if ds == 0:
-            raise ValueError("keep_ds needs bfloat16, head_dim 128 and causal self-attention with Lq == Lk a multiple of 256")
+            raise ValueError(_KEEP_DS_SHAPES)
         n += ds
     return torch.empty(n, dtype=torch.uint8, device=q.device)
+
+
+def attn_bwd_workspace_bytes(q, k, keep_ds: bool = False, causal: bool = True) -> Optional[int]:
+    """Bytes of workspace that attn_bwd needs on these shapes; None if keep_ds is asked for a shape that cannot keep dS."""
+    B, Lq, Hq, D = q.shape
+    lib = _lib.load()
+    n = lib.ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q))
+    if keep_ds:
+        ds = lib.ody_attn_bwd_ds_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q), int(causal))
+        if ds == 0:
+            return None
+        n += ds
+    return n
+
+
+def _shared_bwd_workspace(q, calls):
+    """One workspace for a sequence of attn_bwd calls with the same queries: `calls` is a list of (k, causal).
+    Returns it with the keep_ds setting of every call: on where the shape qualifies and the scratch stays within
+    keep_ds_max_bytes(), all off if that much memory is not there."""
+    B, Lq, Hq, D = q.shape
+    lib = _lib.load()
+    base = [lib.ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q)) for k, _ in calls]
+    ds = [lib.ody_attn_bwd_ds_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q), int(c)) for k, c in calls]
+    limit = keep_ds_max_bytes(q.device)
+    keeps = [0 < d <= limit for d in ds]
+    if any(keeps):
+        try:
+            n = max(b + (d if kp else 0) for b, d, kp in zip(base, ds, keeps))
+            return torch.empty(n, dtype=torch.uint8, device=q.device), keeps
+        except torch.OutOfMemoryError:
+            pass
+    return torch.empty(max(base), dtype=torch.uint8, device=q.device), [False] * len(calls)
 
 
 def cast_from_f32(src, dtype) -> torch.Tensor:
@@ -579,12 +612,12 @@ class RingBlocksAttnFunc(torch.autograd.Function):
         # Q / dO images depend on the queries only and are built by the first block's call
         dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
         same_kv_shape = all(k.shape == ks[0].shape for k in ks)
-        ws = attn_bwd_workspace(q, max(ks, key=lambda t: t.shape[1])) if nb else None
+        ws, keeps = _shared_bwd_workspace(q, [(ks[b], b == ctx.causal_block) for b in range(nb)]) if nb else (None, [])
         dks, dvs = [], []
         for b in range(nb):
             _, dk, dv = attn_bwd(q, ks[b], vs[b], out, lse, dout, causal=(b == ctx.causal_block),
                                  scale=ctx.softmax_scale, dq=dq, accumulate_dq=(b > 0), workspace=ws,
-                                 reuse_query_side=(b > 0 and same_kv_shape))
+                                 reuse_query_side=(b > 0 and same_kv_shape), keep_ds=keeps[b])
             dks.append(dk)
             dvs.append(dv)
         return (cast_from_f32(dq, q.dtype), None, None, *dks, *dvs)
@@ -658,16 +691,20 @@ class ZigzagRingRankAttnFunc(torch.autograd.Function):
             dout = dout.contiguous()
         dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
         lse_b = lse[:, :, c:].contiguous()
-        ws = attn_bwd_workspace(q, ks[0])
+        steps = list(ZigzagRingRankAttnFunc._steps(ctx.rank, world))
+        # sized for the largest step (both query chunks against both key chunks); a step with fewer queries asks for less
+        ws, _ = _shared_bwd_workspace(q, [(ks[0], False)])
         dks = [torch.zeros_like(k) for k in ks]
         dvs = [torch.zeros_like(v) for v in vs]
         prev = None
-        for s, ((q0, q1), (k0, k1), causal) in enumerate(ZigzagRingRankAttnFunc._steps(ctx.rank, world)):
+        for s, ((q0, q1), (k0, k1), causal) in enumerate(steps):
             qs, kr = slice(q0 * c, q1 * c), slice(k0 * c, k1 * c)
             kind = (q0, q1, k0, k1)
+            need = attn_bwd_workspace_bytes(q[:, qs], ks[s][:, kr], True, causal)
             attn_bwd(q[:, qs], ks[s][:, kr], vs[s][:, kr], out[:, qs], lse if q1 - q0 == 2 else lse_b, dout[:, qs],
                      causal=causal, scale=ctx.softmax_scale, dq=dq[:, qs], dk=dks[s][:, kr], dv=dvs[s][:, kr],
-                     accumulate_dq=(s > 0), workspace=ws, reuse_query_side=(kind == prev))
+                     accumulate_dq=(s > 0), workspace=ws, reuse_query_side=(kind == prev),
+                     keep_ds=(need is not None and need <= ws.numel()))
             prev = kind
         return (cast_from_f32(dq, q.dtype), None, None, None, *dks, *dvs)
 

@@ -250,8 +250,9 @@ def test_attention_bwd_kept_ds_policy(dev):
     shape that does not qualify is an error; the C ABI refuses a workspace without room for dS."""
     from odysseus_transformer_amd import ops, _lib
     lib = _lib.load()
-    assert lib.ody_attn_bwd_ds_bytes(1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 1) == 2 * 3 * 128 * 1024
-    for args in ((1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 0), (1, 500, 500, 2, 2, 128, _lib.ODY_BF16, 1),
+    assert lib.ody_attn_bwd_ds_bytes(1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 1) == 2 * 3 * 128 * 1024   # 3 blocks per head
+    assert lib.ody_attn_bwd_ds_bytes(1, 512, 768, 2, 2, 128, _lib.ODY_BF16, 0) == 2 * 6 * 128 * 1024   # 2 x 3 blocks
+    for args in ((1, 500, 500, 2, 2, 128, _lib.ODY_BF16, 1), (1, 512, 700, 2, 2, 128, _lib.ODY_BF16, 0),
                  (1, 512, 768, 2, 2, 128, _lib.ODY_BF16, 1), (1, 512, 512, 2, 2, 64, _lib.ODY_BF16, 1),
                  (1, 512, 512, 2, 2, 128, _lib.ODY_F32, 1)):
         assert lib.ody_attn_bwd_ds_bytes(*args) == 0, args
@@ -280,3 +281,27 @@ def test_attention_bwd_kept_ds_policy(dev):
     small = ops.attn_bwd_workspace(q, k)
     with pytest.raises(ValueError):
         ops.attn_bwd(q, k, v, o, lse, do, causal=True, workspace=small, keep_ds=True)
+
+
+@pytest.mark.parametrize("case", [(1, 512, 768, 2, 2), (2, 768, 256, 4, 2), (1, 256, 1024, 4, 1)],
+                         ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d" % c)
+def test_attention_bwd_kept_ds_full_blocks(case, dev):
+    """Kept dS for a fully visible block of keys (a ring step): any whole number of 256-row blocks on either side,
+    and the running fp32 dq that such a step adds into."""
+    from odysseus_transformer_amd import ops
+    B, Lq, Lk, Hq, Hkv = case
+    print(f"case={case}", flush=True)
+    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, 128, torch.bfloat16, seed=Lq + Lk)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=False)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float(), causal=False)
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=False)
+    acc0 = randn((B, Lq, Hq, 128), 6).to(dev)
+    acc = acc0.clone()
+    _, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=False, dq=acc, accumulate_dq=True, keep_ds=True)
+    assert_parity((acc - acc0).cpu(), dq_ref, TOL_BF16, "dq added to an fp32 buffer", 1e-3)
+    assert_parity(dk, dk_ref, TOL_BF16, "dk", 1e-3)
+    assert_parity(dv, dv_ref, TOL_BF16, "dv")
+    dq2, dk2, dv2 = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=False, keep_ds=False)
+    assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
+    assert_parity(dq2, dq_ref, TOL_BF16, "dq of the recomputing kernel", 1e-3)
