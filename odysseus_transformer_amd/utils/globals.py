@@ -2,8 +2,9 @@
 
 One flat allocation per (name, dtype) key that only ever grows; `get_tensor` hands out a
 view of its head.  Two tensors of one key alias each other: a caller holds at most one at a
-time.  Sized for a 288 GB device: the largest user here is the gathered (L, d) activation,
-256 MiB at L = 32768, d = 4096.
+time.  Sized for a 288 GB device: the largest users here are the attention backward's kept dS
+(4 GiB at 4 heads x 32768 tokens) and the gathered (L, d) activation (256 MiB at L = 32768,
+d = 4096).
 """
 from __future__ import annotations
 
