@@ -19,11 +19,11 @@ from sampled import edge_samples, sampled_checks
 pytestmark = pytest.mark.gpu
 
 
-def run_attention(q, k, v, do, dev, causal=True):
+def run_attention(q, k, v, do, dev, causal=True, keep_ds=None):
     from odysseus_transformer_amd import ops
     qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
     o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
-    dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal)
+    dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=keep_ds)
     torch.cuda.synchronize()
     return tuple(t.cpu() for t in (o, lse, dq, dk, dv))
 
@@ -46,6 +46,10 @@ def test_cfg2_shard_whole_result(dev):
     again = run_attention(q, k, v, do, dev)
     for a, b in zip((o, lse, dq, dk, dv), again):
         assert torch.equal(a, b)
+    # the default at this shape keeps dS for the dQ kernel; the recomputing dQ kernel on the same inputs
+    _, _, dq_r, dk_r, dv_r = run_attention(q, k, v, do, dev, keep_ds=False)
+    assert_parity(dq_r, dq_ref, TOL_BF16, "dq of the recomputing kernel")
+    assert torch.equal(dk_r, dk) and torch.equal(dv_r, dv)
 
 
 @pytest.mark.parametrize("L,Hq,Hkv", [(131072, 4, 4), (65536, 4, 1)], ids=["cfg3_L131072", "cfg4_L65536_gqa4"])
