@@ -72,6 +72,11 @@ __global__ __launch_bounds__(FW_THREADS) void attn_fwd_w8_kernel(const AttnParam
     if (qi < p.Lq) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + (int64_t)qi * p.sq.l + 16 * ks + 8 * g);
     else qf[ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
   }
+  // Q^T must have ARRIVED before the loop: left pending, the compiler places its wait for these register loads at
+  // their first use, inside the loop, as a wait for every load in flight -- and the ring's direct loads, which are
+  // issued two turns ahead, would have to land within one.
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++) asm volatile("" : "+v"(qf[ks]));
   const int lim = p.causal ? min(p.Lk - 1, qi + p.off) : p.Lk - 1;   // last key this lane's query sees
   const float c2 = p.scale_log2e;
   const int rbase = row_frag_base(g, i), ibase = image_frag_base(g, i);
