@@ -61,26 +61,6 @@ int ody_device_info(int* compute_units, int* clock_khz, int* lds_bytes_per_cu);
 int ody_profile_enable(int on);
 int ody_profile_collect(char* out, size_t cap);
 
-/* Measurement aid (no counterpart in the reference): a loop of nothing but bf16 32x32x16 MFMAs on
- * register operands taken from `operands` (at least 1 MiB of bf16 on the device), 4 wavefronts per
- * block, 16 * iters MFMAs per wavefront, 32768 FLOP each.  What it sustains with the operand data
- * of interest is the rate the matrix pipe can actually be driven at -- with random data well below
- * the published peak, which only constant operands reach.  sink: blocks * 256 floats.
- */
-int ody_mfma_probe(const void* operands, float* sink, int blocks, int iters, void* stream);
-
-/* Measurement aid (no counterpart in the reference): what each ingredient of an attention tile costs on
- * top of the bare MFMAs.  Workgroups of 8 wavefronts (two per SIMD, 96 KB of LDS: one per CU), a barrier
- * per turn, 32 MFMAs per wavefront and turn; `what` adds the vector work of a 32 x 64 score tile
- * (ODY_PROBE_VECTOR), the MFMA A operands read from LDS (ODY_PROBE_LDS_READS) and 32 KB of direct
- * global->LDS loads per turn and workgroup, two turns ahead (ODY_PROBE_DIRECT_LOADS, from the 64 MiB at
- * stream_src).  Built combinations: 0, 1, 3, 5, 7.  operands: at least 1 MiB of bf16; sink: blocks * 512
- * floats.  FLOP: blocks * 8 * turns * 32 * 32768.
- */
-enum ody_probe_parts { ODY_PROBE_VECTOR = 1, ODY_PROBE_LDS_READS = 2, ODY_PROBE_DIRECT_LOADS = 4 };
-int ody_pipeline_probe(const void* operands, const void* stream_src, float* sink, int blocks, int turns, int what,
-                       void* stream);
-
 /* ---- attention ---------------------------------------------------------
  * Replaces flash_attn_func(q, k, v, dropout_p=0, softmax_scale, causal) as
  * reached from decoder/odysseus.py:256-263 (via HF _flash_attention_forward),
@@ -227,8 +207,11 @@ int ody_gemm(int op, const void* A, const void* B, void* C, const void* bias,
  * ody_linear_dgrad_swiglu d_gate_up (T, 2 I) = SwiGLU backward of (gate_up, dh) with dh = dy (T, K) Wd (K, I):
  *                         the input gradient of the down projection (utils/linear_zero3.py:68) feeding the
  *                         backward of decoder/odysseus.py:295; dh itself is never stored.  workspace:
- *                         ody_linear_dgrad_swiglu_workspace_bytes(...) bytes (0 when the fused kernel applies;
- *                         otherwise room for dh), 16-byte aligned.
+ *                         ody_linear_dgrad_swiglu_workspace_bytes(...) bytes (0 when the shape takes the fused
+ *                         kernel; otherwise room for dh), 16-byte aligned.  The query goes by the shape alone and
+ *                         assumes 16-byte aligned pointers and leading dimensions that are multiples of 8: operands
+ *                         without them take the two-kernel path whatever the shape and need T * I elements of
+ *                         workspace (the call returns ODY_ERR_WORKSPACE and says so if it is missing).
  */
 int ody_linear_residual(const void* x, const void* w, const void* residual, void* y, int M, int N, int K,
                         int64_t ldx, int64_t ldw, int64_t ld_res, int64_t ldy, int dtype, void* stream);

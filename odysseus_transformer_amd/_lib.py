@@ -25,8 +25,6 @@ SIGNATURES = {
     "ody_device_info": (_i, [_p, _p, _p]),
     "ody_profile_enable": (_i, [_i]),
     "ody_profile_collect": (_i, [C.c_char_p, _sz]),
-    "ody_mfma_probe": (_i, [_p, _p, _i, _i, _p]),
-    "ody_pipeline_probe": (_i, [_p, _p, _p, _i, _i, _i, _p]),
     "ody_attn_fwd_workspace_bytes": (_sz, [_i] * 7),
     "ody_attn_fwd": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p, _sz, _p]),
     "ody_attn_fwd_noalloc": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p]),

@@ -20,6 +20,9 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 OBJ = CSRC / "build"
 LIB = PKG / "lib" / "libodysseus_hip.so"
+# measurement aids of bench.py (synthetic MFMA / tile-cost probes): their own library, not part of the product's ABI
+BENCH_SRC = CSRC / "bench" / "probes.hip"
+BENCH_LIB = PKG / "lib" / "libodysseus_bench.so"
 INCLUDE = PKG.parent / "include"
 
 HIPCC_FLAGS = [
@@ -68,8 +71,13 @@ def build(force: bool = False, jobs: int = 4, verbose: bool = True) -> Path:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stderr}")
+    if force or _newer(BENCH_SRC, BENCH_LIB, []):
+        cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", "-o", str(BENCH_LIB), str(BENCH_SRC)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {BENCH_SRC.name}:\n{r.stderr}")
     if verbose:
-        print(f"built {LIB} ({LIB.stat().st_size} bytes) from {len(srcs)} sources")
+        print(f"built {LIB} ({LIB.stat().st_size} bytes) from {len(srcs)} sources, and {BENCH_LIB.name}")
     return LIB
 
 
