@@ -112,25 +112,58 @@ def measured_traffic():
     return json.loads(m.group(1)) if m else {}
 
 
+_PROBES = None
+
+
+def probes():
+    """bench.py's own measurement kernels (odysseus_transformer_amd/lib/libodysseus_bench.so, built beside the product
+    library from csrc/bench/probes.hip): not part of the product's ABI."""
+    global _PROBES
+    if _PROBES is None:
+        import ctypes as C
+        path = ROOT / "odysseus_transformer_amd" / "lib" / "libodysseus_bench.so"
+        if not path.exists():
+            from odysseus_transformer_amd import build
+            build.build(verbose=False)
+        lib = C.CDLL(str(path))
+        lib.ody_bench_mfma_probe.restype = C.c_int
+        lib.ody_bench_mfma_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        lib.ody_bench_pipeline_probe.restype = C.c_int
+        lib.ody_bench_pipeline_probe.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        _PROBES = lib
+    return _PROBES
+
+
+def _probe(name, *args):
+    rc = getattr(probes(), name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed with status {rc}")
+
+
 def mfma_sustained(_lib, dev):
-    """What the matrix pipe sustains in a loop of nothing but MFMAs on register operands: with
-    constant operands (the published peak is reached) and with random ones (what real data allows)."""
+    """What the matrix pipe sustains in a loop of nothing but MFMAs on register operands: with constant operands (the
+    published peak is reached) and with random ones (what real data allows), for the 32x32x16 instruction that the
+    kernels of this library use and for the 16x16x32 one."""
     import torch
-    blocks, iters = 512, 8000            # 8 wavefronts per CU; ~10 ms at the rates seen
+    blocks, iters = 256, 8000            # one block of 4 wavefronts per CU; ~5 ms at the rates seen
     sink = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
     res = {}
     g = torch.Generator().manual_seed(7)
+    st = torch.cuda.current_stream().cuda_stream
     for name, data in (("constant_operands", torch.ones(1 << 19)), ("random_operands", torch.randn(1 << 19, generator=g))):
         ops_ = data.to(torch.bfloat16).to(dev)
-        for _ in range(2):
-            _lib.call("ody_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, 200, torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        _lib.call("ody_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, iters, torch.cuda.current_stream().cuda_stream)
-        e1.record()
-        torch.cuda.synchronize()
-        res[name + "_tflops"] = round(blocks * 4 * iters * 16 * 32768.0 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+        for shape, tag in ((0, ""), (1, "_16x16x32")):
+            best = None
+            for rep in range(3):
+                _probe("ody_bench_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, 200, shape, st)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                _probe("ody_bench_mfma_probe", ops_.data_ptr(), sink.data_ptr(), blocks, iters, shape, st)
+                e1.record()
+                torch.cuda.synchronize()
+                best = e0.elapsed_time(e1) if best is None else min(best, e0.elapsed_time(e1))
+            res[name + tag + "_tflops"] = round(blocks * 4 * iters * 16 * 32768.0 / (best * 1e-3) / 1e12, 1)
     return res
 
 
@@ -153,7 +186,7 @@ def tile_cost_ladder(_lib, dev, fwd_ms):
         for rep in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            _lib.call("ody_pipeline_probe", ops_.data_ptr(), src.data_ptr(), sink.data_ptr(), blocks, turns, what, st)
+            _probe("ody_bench_pipeline_probe", ops_.data_ptr(), src.data_ptr(), sink.data_ptr(), blocks, turns, what, st)
             e1.record()
             torch.cuda.synchronize()
             if rep:
@@ -264,6 +297,11 @@ def main():
                      dv=dqkv[:, :, H + HKV:])
         state["o"] = o
 
+    # Kept dS is opt-in (it spends B * Hq * L * L bytes of scratch: 4 GiB here, 64 GiB at L = 131072): the benchmark
+    # opts in, with a quarter of the device's memory as its budget, and also times the step without it below.
+    ds_budget = prop.total_memory // 4
+    ops.set_keep_ds_max_bytes(ds_budget)
+    ds_bytes = _lib.load().ody_attn_bwd_ds_bytes(1, L, L, H, HKV, D, _lib.ODY_BF16, 1)
     for _ in range(a.warmup):
         step()
     if a.copy_probe:
@@ -287,6 +325,10 @@ def main():
     prof = _lib.profile_collect()
     _lib.profile_enable(False)
     step_spread = spread(time_events(step, a.steps, 0))   # and once more, every step between its own pair of events
+    # ---- the same step on the recomputing backward (no dS scratch: what ops.attn_bwd does unless asked otherwise)
+    ops.set_keep_ds_max_bytes(0)
+    sec_recompute = time_gpu(step, a.steps, 3)
+    ops.set_keep_ds_max_bytes(ds_budget)
 
     f_fwd, f_bwd = attn_flops(L, L, H, D)
     # algorithmic FLOPs per launch: the backward's 5 tile products are S, dP, dV, dK (in the
@@ -335,7 +377,12 @@ def main():
         "config": {"workload": "causal attention fwd+bwd, Llama-2-7B rank shard at N=8: 4 heads x 128, L=32768, "
                                "batch 1 (attention part of the 32768-token bf16 configuration)",
                    "heads": H, "kv_heads": HKV, "head_dim": D, "seq_len": L, "flops_per_step": f_fwd + f_bwd,
-                   "seeds": {"qkv": 2001, "dout": 2002}},
+                   "seeds": {"qkv": 2001, "dout": 2002},
+                   "backward": "kept dS" if dq_kernel == "attn_bwd_dq_kept" else "recomputing",
+                   "ds_scratch_bytes": ds_bytes if dq_kernel == "attn_bwd_dq_kept" else 0,
+                   "keep_ds_budget_bytes": ds_budget},
+        "ms_per_step_recompute": round(sec_recompute * 1e3, 4),
+        "value_recompute": round((f_fwd + f_bwd) / sec_recompute / 1e12, 2),
         "step_ms": step_spread, "fwd_ms": round(fwd_ms, 4), "bwd_ms": round(bwd_ms, 4),
         "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 1), "bwd_tflops": round(f_bwd / (bwd_ms * 1e-3) / 1e12, 1),
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
@@ -659,10 +706,10 @@ def power_under_load(_lib, ops, dev, attention_step):
     return {
         "attention_step": under(attention_step),
         "gemm_nt_8192": under(lambda: ops.gemm(ops.GEMM_NT, a, b)),
-        "mfma_probe_random_operands": under(lambda: _lib.call("ody_mfma_probe", rand.data_ptr(), sink.data_ptr(), 4096,
-                                                              2000, st)),
-        "mfma_probe_constant_operands": under(lambda: _lib.call("ody_mfma_probe", ones.data_ptr(), sink.data_ptr(),
-                                                                4096, 2000, st)),
+        "mfma_probe_random_operands": under(lambda: _probe("ody_bench_mfma_probe", rand.data_ptr(), sink.data_ptr(), 4096,
+                                                              2000, 0, st)),
+        "mfma_probe_constant_operands": under(lambda: _probe("ody_bench_mfma_probe", ones.data_ptr(), sink.data_ptr(),
+                                                                4096, 2000, 0, st)),
         "copy_512MiB": under(lambda: dst.copy_(src)),
     }
 

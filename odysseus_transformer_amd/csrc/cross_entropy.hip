@@ -69,7 +69,9 @@ __global__ __launch_bounds__(256) void ce_fwd_kernel(const T* __restrict__ logit
     const int64_t lab = labels[row];
     const bool valid = lab != ignore_index && lab >= 0 && lab < V;
     lse_out[row] = lse;
-    losses[row] = valid ? lse - (float)x[lab] : 0.f;
+    // a label outside [0, V) that is not ignore_index is a bug upstream (a vocabulary off by one, say): its loss is
+    // NaN, and so is every mean or sum it enters, instead of a token silently left out
+    losses[row] = valid ? lse - (float)x[lab] : (lab == ignore_index ? 0.f : __builtin_nanf(""));
   }
 }
 
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(1024) void ce_reduce_kernel(const float* __restrict
   float s = 0.f, c = 0.f;
   for (int t = threadIdx.x; t < T; t += 1024) {
     const int64_t lab = labels[t];
-    if (lab != ignore_index && lab >= 0 && lab < V) s += losses[t], c += 1.f;
+    if (lab != ignore_index) s += losses[t], c += 1.f;   // a label out of range counts, with its NaN
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64), c += __shfl_xor(c, o, 64);

@@ -15,6 +15,7 @@ keywords, parameter names and shapes, and return convention.
 from __future__ import annotations
 
 import inspect
+import warnings
 import math
 from typing import Optional
 
@@ -193,6 +194,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
         computes when the gather is the identity (one rank), there is no bias and autocast asks for no cast;
         the fused kernels exist for bfloat16 and head_dim 128."""
         return (self.fuse_rope and self.head_dim == 128 and get_model_parallel_world_size() == 1
+                and not _has_hooks(self.qkv_proj)
                 and self.qkv_proj.bias is None and hidden_states.dtype == torch.bfloat16
                 and self.qkv_proj.weight.dtype == torch.bfloat16 and hidden_states.is_cuda
                 and not torch.is_autocast_enabled("cuda"))
@@ -202,6 +204,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
         reduce-scatter is the identity (one rank), there is no bias (it is added after the scatter) and
         autocast does not ask for a cast."""
         return (get_model_parallel_world_size() == 1 and self.o_proj.bias is None and self.o_proj.input_is_parallel
+                and not _has_hooks(self.o_proj)
                 and residual.dtype == attn_output.dtype == self.o_proj.weight.dtype
                 and not torch.is_autocast_enabled("cuda"))
 
@@ -242,6 +245,7 @@ class LlamaMLPZeRO(nn.Module):
         w1, w2 = self.gate_up_proj.weight, self.down_proj.weight
         fusable = (get_model_parallel_world_size() == 1 and self.gate_up_proj.bias is None and self.down_proj.bias is None
                    and x.dtype == w1.dtype == w2.dtype and (residual is None or residual.dtype == x.dtype)
+                   and not _has_hooks(self.gate_up_proj, self.down_proj)
                    and not torch.is_autocast_enabled("cuda"))
         if fusable and self.fuse_elementwise:
             return ops.SwiGLUMLPResidualFunc.apply(x, w1, w2, residual)
@@ -282,8 +286,17 @@ class OdysseusDecoderLayer(nn.Module):
         self.self_attn.fuse_rope = fused
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, eps)
+        # set by model.gradient_checkpointing_enable() on a host's layers (the reference's --grad-checkpoint,
+        # train.py:163-164): in training the layer keeps its input only and runs its forward again in backward
+        self.gradient_checkpointing = False
 
     def forward(self, hidden_states, attention_mask=None, position_ids=None, **kwargs):
+        if self.gradient_checkpointing and self.training and torch.is_grad_enabled():
+            from torch.utils.checkpoint import checkpoint
+            return checkpoint(self._forward, hidden_states, attention_mask, position_ids, use_reentrant=False, **kwargs)
+        return self._forward(hidden_states, attention_mask, position_ids, **kwargs)
+
+    def _forward(self, hidden_states, attention_mask=None, position_ids=None, **kwargs):
         # what a host model hands its decoder layers besides (a cache to fill during a prefill)
         cache = {k: kwargs[k] for k in ("past_key_value", "past_key_values", "cache_position") if kwargs.get(k) is not None}
         if self.fused:
@@ -299,6 +312,13 @@ class OdysseusDecoderLayer(nn.Module):
         residual = hidden_states
         hidden_states = self.mlp(self.post_attention_layernorm(hidden_states))
         return residual + hidden_states
+
+
+def _has_hooks(*modules) -> bool:
+    """A fused path reads a projection's weight and never calls the module: forward hooks (or pre-hooks) that
+    someone registered on it would be skipped without notice, so their presence sends the call down the
+    module-by-module path."""
+    return any(m is not None and (m._forward_hooks or m._forward_pre_hooks) for m in modules)
 
 
 def _host_layer_unpacks_two(layer) -> bool:
@@ -328,9 +348,10 @@ def _host_builds_no_mask(model) -> None:
     cfg = getattr(model, "config", None)
     if cfg is not None and getattr(cfg, "_attn_implementation", None) not in (None, "flash_attention_2"):
         try:
-            cfg._attn_implementation = "flash_attention_2"
-        except Exception:   # a host that validates the assignment: the mask check in forward() still guards
-            pass
+            cfg._attn_implementation = "flash_attention_2"   # this model's config only; nothing process-wide
+        except Exception as e:   # a host that validates the assignment: the mask check in forward() still guards
+            warnings.warn(f"could not declare flash_attention_2 in the model's config ({e!r}); the host may hand the "
+                          "modules a dense mask, which they refuse")
 
 
 def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True, fuse_layers=False):
@@ -359,6 +380,7 @@ def apply_odysseus_attn_patch_llama(model, use_zero3_linear=True, fuse_layers=Fa
             for attr in ("attention_type", "gradient_checkpointing"):
                 if hasattr(old, attr):
                     setattr(new, attr, getattr(old, attr))
+            new.gradient_checkpointing = bool(getattr(new, "gradient_checkpointing", False))
             model.model.layers[i] = new
         print("Applied Odysseus patch for LlamaDecoderLayer")
         return

@@ -49,3 +49,16 @@ def hip_zigzag_ring_attention_forward(module, query, key, value, attention_mask,
 def apply_zigzag_ring_attn_monkey_patch_llama(model=None) -> None:
     """decoder/ring.py:98-104.  Pass the model so that its config asks for the flash-attention entry."""
     install_hip_flash_attention(hip_zigzag_ring_attention_forward, model)
+
+
+def apply_zigzag_ring_attn_monkey_patch_mistral(model=None) -> None:
+    """decoder/ring.py:107-113: the same routing for a Mistral host.  The reference assigns to
+    MistralFlashAttention2._flash_attention_forward; the installed transformers reaches every model family's
+    flash-attention call through one registry, so the entry is the one the Llama patch installs.  A Mistral
+    config with a sliding window is refused at the call, as the reference does (decoder/ring.py:29)."""
+    install_hip_flash_attention(hip_zigzag_ring_attention_forward, model)
+
+
+# the names the reference's train.py imports (train.py:23)
+apply_zigzag_ring_attn_patch_llama = apply_zigzag_ring_attn_monkey_patch_llama
+apply_zigzag_ring_attn_patch_mistral = apply_zigzag_ring_attn_monkey_patch_mistral

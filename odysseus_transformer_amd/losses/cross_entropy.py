@@ -79,7 +79,12 @@ class CrossEntropyLoss(nn.Module):
     """Constructor keywords as flash_attn's module.  inplace_backward=True writes the gradient over
     the logits' own storage in backward (the logits are dead after the loss in a training step),
     saving one (tokens, vocab) allocation.  Label smoothing, the z-loss and vocabulary-parallel
-    logits (process_group) are not implemented; the training loop uses none of them."""
+    logits (process_group) are not implemented; the training loop uses none of them.
+
+    Labels: `ignore_index` leaves a token out (loss 0, gradient row 0, not counted in the mean).  Any other
+    label outside [0, vocab) gives that token the loss NaN, which every reduction then shows (its gradient row
+    is 0: the kernels never index out of the row).  One deviation from flash_attn's module: the mean over ZERO
+    counted tokens is 0 here, not the NaN of 0 / 0."""
 
     def __init__(self, ignore_index=-100, reduction="mean", label_smoothing=0.0, lse_square_scale=0.0,
                  inplace_backward=False, process_group=None):

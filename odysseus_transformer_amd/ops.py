@@ -123,9 +123,10 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
 
     keep_ds spends scratch memory to save arithmetic: the dK/dV kernel keeps dS (2 bytes per visible
     query-key pair: about B * Hq * L * L bytes when causal) and dQ becomes one product over it instead of a second
-    pass over S and dP.  bfloat16, head_dim 128, Lq and Lk multiples of 256, causal only with Lq == Lk.  None (the
-    default) turns it on where the shape qualifies, no `workspace` is passed and the scratch stays within
-    keep_ds_max_bytes(); True insists (ValueError where the shape does not qualify); False never."""
+    pass over S and dP.  bfloat16, head_dim 128, Lq and Lk multiples of 256, causal only with Lq == Lk.  It is
+    opt-in: None (the default) turns it on only where the shape qualifies, no `workspace` is passed and the
+    scratch stays within the budget of set_keep_ds_max_bytes() / ODYSSEUS_KEEP_DS_MAX_BYTES (0 unless set) or is
+    already there in the arena; True insists (ValueError where the shape does not qualify); False never."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
@@ -150,12 +151,13 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
         raise ValueError(_KEEP_DS_SHAPES)
     ws = None
     if keep_ds is None:
-        keep_ds = workspace is None and 0 < ds_bytes <= keep_ds_max_bytes(q.device)
+        keep_ds = workspace is None and _keep_ds_fits(ws_bytes, ds_bytes, q.device)
         if keep_ds:
             try:
                 ws = scratch(ws_bytes + ds_bytes, "attn_bwd_workspace", q.device)
-            except torch.OutOfMemoryError:   # the memory is not there: the recomputing kernels need none of it
-                keep_ds = False
+            except torch.OutOfMemoryError:   # the memory is not there: the recomputing kernels need none of it,
+                keep_ds = False              # and this size is not tried again (the allocator's retry synchronises)
+                _KEEP_DS_OOM[str(q.device)] = min(ds_bytes, _KEEP_DS_OOM.get(str(q.device), 1 << 62))
     if keep_ds:
         ws_bytes += ds_bytes
     if workspace is None:
@@ -189,24 +191,53 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
 
 
 _KEEP_DS_MAX_BYTES: Optional[int] = None
+_KEEP_DS_OOM: dict = {}   # device -> smallest dS scratch whose allocation failed there (never tried again at or above it)
 _KEEP_DS_SHAPES = "keep_ds needs bfloat16, head_dim 128, Lq and Lk multiples of 256 and, if causal, Lq == Lk"
 
 
 def keep_ds_max_bytes(device=None) -> int:
-    """Largest dS scratch that attn_bwd takes on its own (keep_ds=None): set_keep_ds_max_bytes(), else the
-    environment variable ODYSSEUS_KEEP_DS_MAX_BYTES, else a quarter of the device's memory."""
+    """Largest dS scratch that attn_bwd takes on its own (keep_ds=None).  Kept dS is opt-in -- it holds about
+    B * Hq * L * L bytes for the life of the arena (4 GiB at 4 heads x 32768 tokens, 64 GiB at L = 131072) for a
+    few percent of speed: set_keep_ds_max_bytes(), else the environment variable ODYSSEUS_KEEP_DS_MAX_BYTES, else 0.
+    Scratch that the arena's "attn_bwd_workspace" buffer already holds is used whatever the limit says: it costs
+    nothing more."""
     if _KEEP_DS_MAX_BYTES is not None:
         return _KEEP_DS_MAX_BYTES
     env = os.environ.get("ODYSSEUS_KEEP_DS_MAX_BYTES")
     if env is not None:
         return int(env)
-    return torch.cuda.get_device_properties(device).total_memory // 4
+    return 0
 
 
 def set_keep_ds_max_bytes(nbytes: Optional[int]) -> None:
-    """0 turns the automatic use of keep_ds off; None restores the default."""
+    """The budget of kept dS for calls that leave keep_ds=None; 0 turns it off, None restores the default (off unless
+    ODYSSEUS_KEEP_DS_MAX_BYTES says otherwise)."""
     global _KEEP_DS_MAX_BYTES
     _KEEP_DS_MAX_BYTES = nbytes
+    _KEEP_DS_OOM.clear()
+
+
+def _arena_holds(name: str, device) -> int:
+    """Bytes that the arena's uint8 buffer `name` already holds on `device` (0 without an arena)."""
+    from .utils import globals as _globals
+    arena = _globals._Arena.instance
+    if arena is None:
+        return 0
+    adev = torch.device(arena.dev)
+    if adev.type != device.type or (adev.index is not None and adev.index != device.index):
+        return 0
+    backing = arena.buffer.get((name, torch.uint8))
+    return 0 if backing is None else backing.numel()
+
+
+def _keep_ds_fits(ws_bytes: int, ds_bytes: int, device) -> bool:
+    """The policy of keep_ds=None: within the budget (and not a size that already failed to allocate on this device),
+    or free because the arena's buffer is that large already."""
+    if ds_bytes <= 0:
+        return False
+    if ws_bytes + ds_bytes <= _arena_holds("attn_bwd_workspace", device):
+        return True
+    return ds_bytes <= keep_ds_max_bytes(device) and ds_bytes < _KEEP_DS_OOM.get(str(device), 1 << 62)
 
 
 def attn_bwd_workspace(q, k, keep_ds: bool = False, causal: bool = True) -> torch.Tensor:
@@ -245,13 +276,14 @@ def _shared_bwd_workspace(q, calls):
     base = [lib.ody_attn_bwd_workspace_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q)) for k, _ in calls]
     ds = [lib.ody_attn_bwd_ds_bytes(B, Lq, k.shape[1], Hq, k.shape[2], D, _dt(q), int(c)) for k, c in calls]
     limit = keep_ds_max_bytes(q.device)
-    keeps = [0 < d <= limit for d in ds]
+    failed = _KEEP_DS_OOM.get(str(q.device), 1 << 62)
+    keeps = [0 < d <= limit and d < failed for d in ds]
     if any(keeps):
         try:
             n = max(b + (d if kp else 0) for b, d, kp in zip(base, ds, keeps))
             return torch.empty(n, dtype=torch.uint8, device=q.device), keeps
         except torch.OutOfMemoryError:
-            pass
+            _KEEP_DS_OOM[str(q.device)] = min(failed, min(d for d, kp in zip(ds, keeps) if kp))
     return torch.empty(max(base), dtype=torch.uint8, device=q.device), [False] * len(calls)
 
 
@@ -346,9 +378,19 @@ def linear_residual(x, weight, residual):
 _ROPE_TABLE_LAST = None   # (position tensor, its version, rows, head_dim, base, device, stream, table) of the last table built
 
 
+def _tensor_version(t) -> int:
+    """The autograd version counter of `t`; inference tensors (torch.inference_mode) have none and cannot be
+    modified in place outside that mode: -1."""
+    try:
+        return t._version
+    except RuntimeError:
+        return -1
+
+
 def rope_table(position_ids, rows: int, head_dim: int, base: float = 10000.0, device=None, inv_freq=None) -> torch.Tensor:
     """(rows, head_dim) bfloat16: [r, 2 j] = cos, [r, 2 j + 1] = sin of position r times frequency j, rounded
-    as rope_ rounds them.  position_ids: int64 with `rows` elements in the order of the rows, or None for arange.
+    as rope_ rounds them.  position_ids: int64 with `rows` elements in the order of the rows -- or with rows / B
+    elements, one sequence that every batch entry shares, e.g. (1, L) for (B, L) rows -- or None for arange.
 
     The layers of a model are handed one and the same position tensor: the last table is kept and returned again
     for the same tensor object (unmodified since), shape, base and stream.  Treat the result as read-only."""
@@ -360,14 +402,18 @@ def rope_table(position_ids, rows: int, head_dim: int, base: float = 10000.0, de
     if device is None:
         raise ValueError("rope_table needs position_ids or a device")
     device = torch.device(device)
-    key = (None if pos_arg is None else pos_arg._version, rows, head_dim, float(base), str(device), _stream())
+    key = (None if pos_arg is None else _tensor_version(pos_arg), rows, head_dim, float(base), str(device), _stream())
     last = _ROPE_TABLE_LAST
     if inv_freq is None and last is not None and last[0] is pos_arg and last[1] == key:
         return last[2]
     if position_ids is not None:
-        position_ids = position_ids.to(torch.int64).reshape(-1).contiguous()
-        if position_ids.numel() != rows:
-            raise ValueError(f"{position_ids.numel()} positions for {rows} rows")
+        position_ids = position_ids.to(torch.int64).reshape(-1)
+        n = position_ids.numel()
+        if n != rows:
+            if n == 0 or rows % n:
+                raise ValueError(f"{n} positions for {rows} rows")
+            position_ids = position_ids.repeat(rows // n)     # one sequence shared by the batch
+        position_ids = position_ids.contiguous()
     custom_freq = inv_freq is not None
     if inv_freq is None:
         inv_freq = rope_inv_freq(head_dim, base, device)
@@ -423,6 +469,10 @@ def linear_dgrad_swiglu(dy, w_down, gate_up):
                          f"{tuple(gate_up.shape)} {gate_up.dtype} do not fit")
     dgu = torch.empty((T, 2 * I), dtype=dy.dtype, device=dy.device)
     ws_bytes = _lib.load().ody_linear_dgrad_swiglu_workspace_bytes(T, I, K, _dt(dy))
+    if ws_bytes == 0 and any(t.data_ptr() % 16 or t.stride(0) % 8 for t in (dy, w_down, gate_up, dgu)):
+        # the size query goes by the shape alone; the one-kernel path also wants 16-byte aligned rows, and a
+        # column-sliced view without them takes the two-kernel path, which keeps dh (T, I) in a workspace
+        ws_bytes = (T * I * dy.element_size() + 255) & ~255
     ws = scratch(ws_bytes, "dgrad_swiglu_workspace", dy.device) if ws_bytes else None
     _lib.call("ody_linear_dgrad_swiglu", dy.data_ptr(), w_down.data_ptr(), gate_up.data_ptr(), dgu.data_ptr(), T, I, K,
               _rowmajor2d(dy, "dy"), _rowmajor2d(w_down, "w_down"), _rowmajor2d(gate_up, "gate_up"), dgu.stride(0),
@@ -823,10 +873,9 @@ class QKVRoPEAttnFunc(torch.autograd.Function):
         B, L, K = x.shape
         x2 = x.reshape(B * L, K)
         x2 = x2 if x2.stride(1) == 1 else x2.contiguous()
-        pos = position_ids
-        if pos is not None and pos.numel() != B * L:
-            pos = pos.expand(B, L)
-        table = rope_table(pos, B * L, head_dim, rope_base, device=x.device)
+        # the tensor as the caller handed it over: every layer passes the same object, which is what the table's
+        # cache goes by (a (1, L) tensor serves all B batch entries)
+        table = rope_table(position_ids, B * L, head_dim, rope_base, device=x.device)
         H = n_heads + 2 * n_kv_heads
         qkv = linear_rope(x2, weight, table, n_heads + n_kv_heads, head_dim).view(B, L, H, head_dim)
         a, b = n_heads, n_heads + n_kv_heads

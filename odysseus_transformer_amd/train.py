@@ -97,6 +97,40 @@ def build_model(args, dev):
     return model
 
 
+def init_prof(use_profiler: bool, out_dir: str = "./profile/"):
+    """The reference's profiler context (train.py:28-46): two warm-up and four recorded steps of device activity,
+    written as a trace for TensorBoard under ./profile/; a null context without the flag.  Under rocprofv3 leave the
+    flag off: every step also opens a named range (torch.profiler.record_function "train_step_<n>") either way."""
+    from contextlib import nullcontext
+    if not use_profiler:
+        return nullcontext()
+    return torch.profiler.profile(
+        activities=[torch.profiler.ProfilerActivity.CUDA],
+        schedule=torch.profiler.schedule(wait=0, warmup=2, active=4, repeat=1),
+        on_trace_ready=torch.profiler.tensorboard_trace_handler(out_dir),
+        record_shapes=True, with_stack=True)
+
+
+def enable_grad_checkpoint(model) -> int:
+    """--grad-checkpoint (train.py:163-164 calls model.gradient_checkpointing_enable()): every decoder layer's
+    activations are dropped after the forward pass and recomputed in backward.  The host model switches its own
+    layers on; layers that the patch replaced (OdysseusDecoderLayer) get the same flag.  Returns the number of
+    checkpointed layers."""
+    from .decoder.odysseus import OdysseusDecoderLayer
+    try:
+        model.gradient_checkpointing_enable(gradient_checkpointing_kwargs={"use_reentrant": False})
+    except Exception as e:   # a host without that switch: the library's own layers below still checkpoint
+        print(f"gradient_checkpointing_enable() of the host model failed: {e!r}")
+    n = 0
+    for layer in model.model.layers:
+        if isinstance(layer, OdysseusDecoderLayer):
+            layer.gradient_checkpointing = True
+            n += 1
+        elif getattr(layer, "gradient_checkpointing", False):
+            n += 1
+    return n
+
+
 def main(args) -> dict:
     from .decoder.odysseus import apply_odysseus_attn_patch_llama
     from .decoder.tensor_parallel import apply_tpsp_attn_patch_llama
@@ -142,6 +176,12 @@ def main(args) -> dict:
                 m.weight.normal_(0.0, 0.02)
     if args.native_host_modules:
         use_native_host_modules(model)
+    if args.keep_ds_max_gb > 0:
+        from . import ops
+        ops.set_keep_ds_max_bytes(int(args.keep_ds_max_gb * 1024 ** 3))
+    checkpointed = enable_grad_checkpoint(model) if args.grad_checkpoint else 0
+    if args.grad_checkpoint:
+        print(f"gradient checkpointing on for {checkpointed} decoder layers")
     mem = lambda: (torch.cuda.memory_allocated(dev) / 1024 ** 3, torch.cuda.memory_reserved(dev) / 1024 ** 3)
     print(f"{args.parallel_mode} After init model, CUDA memory allocated: {mem()[0]:.2f} GB, reserved: {mem()[1]:.2f} GB")
 
@@ -158,28 +198,32 @@ def main(args) -> dict:
 
     gen = torch.Generator().manual_seed(args.seed)
     vocab_size = model.config.vocab_size
-    for step in range(args.max_train_steps):
-        if step > warmup_num_iterations:
-            start_time = time.time()
-        batch = torch.randint(vocab_size, size=(1, args.seq_length + 1), generator=gen)
-        input_ids, target_ids = batch[..., :-1], batch[..., 1:]
-        position_ids = torch.arange(args.seq_length).unsqueeze(0).expand(input_ids.shape[0], -1)
-        prepared = prepare_attn_inputs(args.parallel_mode, input_ids, position_ids, target_ids, rank, world_size, dev)
-        logits = model(prepared["local_input_ids"], position_ids=prepared["local_position_ids"], use_cache=False).logits
-        loss = loss_func(logits.reshape(-1, logits.shape[-1]), prepared["local_target_ids"].reshape(-1))
-        print(f"step {step} CUDA memory allocated/reserved: {mem()[0]:.2f}/{mem()[1]:.2f} GB")
-        losses.append(loss.item())
-        print(f"loss {losses[-1]}", flush=True)
-        loss.backward(loss)
-        optim.step()
-        optim.zero_grad()
-        if step >= warmup_num_iterations:
-            # the reference starts and stops its clock without one, so that a timed step pays for the queued tail of the
-            # step before it; here the seven timed steps are seven whole steps
-            torch.cuda.synchronize()
-        if step > warmup_num_iterations:
-            step_times.append(time.time() - start_time)
-            elapse += step_times[-1]
+    with init_prof(args.use_profiler) as prof:
+        for step in range(args.max_train_steps):
+            if step > warmup_num_iterations:
+                start_time = time.time()
+            with torch.profiler.record_function(f"train_step_{step}"):
+                batch = torch.randint(vocab_size, size=(1, args.seq_length + 1), generator=gen)
+                input_ids, target_ids = batch[..., :-1], batch[..., 1:]
+                position_ids = torch.arange(args.seq_length).unsqueeze(0).expand(input_ids.shape[0], -1)
+                prepared = prepare_attn_inputs(args.parallel_mode, input_ids, position_ids, target_ids, rank, world_size, dev)
+                logits = model(prepared["local_input_ids"], position_ids=prepared["local_position_ids"], use_cache=False).logits
+                loss = loss_func(logits.reshape(-1, logits.shape[-1]), prepared["local_target_ids"].reshape(-1))
+                print(f"step {step} CUDA memory allocated/reserved: {mem()[0]:.2f}/{mem()[1]:.2f} GB")
+                losses.append(loss.item())
+                print(f"loss {losses[-1]}", flush=True)
+                loss.backward(loss)
+                optim.step()
+                optim.zero_grad()
+            if step >= warmup_num_iterations:
+                # the reference starts and stops its clock without one, so that a timed step pays for the queued tail of
+                # the step before it; here the seven timed steps are seven whole steps
+                torch.cuda.synchronize()
+            if step > warmup_num_iterations:
+                step_times.append(time.time() - start_time)
+                elapse += step_times[-1]
+            if args.use_profiler:
+                prof.step()
     print(f"{args.parallel_mode} {args.seq_length//1024}K {world_size} Time taken: {elapse:.2f} seconds")
     out = {"parallel_mode": args.parallel_mode, "seq_length": args.seq_length, "layers": model.config.num_hidden_layers,
            "parameters_b": round(total_params / 1e9, 3), "timed_steps": len(step_times), "time_taken_s": round(elapse, 3),
@@ -187,7 +231,8 @@ def main(args) -> dict:
                                                                                       max(elapse, 1e-9), 1),
            "peak_memory_gb": round(torch.cuda.max_memory_allocated(dev) / 1024 ** 3, 2), "losses": [round(l, 4) for l in losses],
            "native_host_modules": bool(args.native_host_modules), "native_optimizer": bool(args.native_optimizer),
-           "fuse_layers": bool(args.fuse_layers and args.parallel_mode == "odysseus")}
+           "fuse_layers": bool(args.fuse_layers and args.parallel_mode == "odysseus"),
+           "grad_checkpoint_layers": checkpointed, "keep_ds_max_gb": args.keep_ds_max_gb}
     print(json.dumps(out))
     return out
 
@@ -201,7 +246,11 @@ def parse_args(argv=None):
     ap.add_argument("--rope-theta", type=float, default=100000)
     ap.add_argument("--model", type=str, default="meta-llama/Llama-2-7b-hf")
     ap.add_argument("--seq-length", type=int, default=16384)
+    ap.add_argument("--grad-checkpoint", action="store_true", default=False,
+                    help="drop every decoder layer's activations after the forward pass and recompute them in backward")
     ap.add_argument("--use_ody_zero3", action="store_true", default=True)
+    ap.add_argument("--use_profiler", action="store_true", default=False,
+                    help="torch.profiler over steps 2-5 (two warm-up, four recorded), trace under ./profile/")
     ap.add_argument("--use_cfg_init_model", action="store_true", default=False)
     ap.add_argument("--parallel_mode", type=str, choices=["odysseus", "ulysses", "dp", "tpsp", "ring"], default="odysseus")
     ap.add_argument("--num-hidden-layers", type=int, default=16, help="16 in the reference's configuration (train.py:71)")
@@ -211,6 +260,10 @@ def parse_args(argv=None):
                          "instead of the attention and MLP modules only, as the reference's patch does")
     ap.add_argument("--native-optimizer", action=argparse.BooleanOptionalAction, default=True,
                     help="AdamW as one HIP kernel per tensor instead of torch.optim.AdamW's element-wise passes")
+    ap.add_argument("--keep-ds-max-gb", type=float, default=0.0,
+                    help="memory the attention backward may spend on kept dS (about Hq * L * L bytes per layer call, one "
+                         "buffer shared by all layers: 8 GiB at 32 heads x 16384 tokens) for a few percent of speed; "
+                         "0 = the recomputing kernels")
     ap.add_argument("--declare-flash-attention", action=argparse.BooleanOptionalAction, default=False,
                     help="set config._attn_implementation before the model is built (needs flash_attn importable); "
                          "the patchers set it afterwards either way")

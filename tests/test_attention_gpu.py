@@ -246,8 +246,8 @@ def test_attention_bwd_kept_ds(case, keep_ds, dev):
 
 
 def test_attention_bwd_kept_ds_policy(dev):
-    """keep_ds=None takes the kept-dS kernels where the shape qualifies and the scratch fits the limit; True on a
-    shape that does not qualify is an error; the C ABI refuses a workspace without room for dS."""
+    """keep_ds=None takes the kept-dS kernels only within a budget the caller set (or in scratch the arena already
+    holds); True on a shape that does not qualify is an error; the C ABI refuses a workspace without room for dS."""
     from odysseus_transformer_amd import ops, _lib
     lib = _lib.load()
     assert lib.ody_attn_bwd_ds_bytes(1, 512, 512, 2, 2, 128, _lib.ODY_BF16, 1) == 2 * 3 * 128 * 1024   # 3 blocks per head
@@ -268,13 +268,26 @@ def test_attention_bwd_kept_ds_policy(dev):
         finally:
             _lib.profile_enable(False)
 
-    assert "attn_bwd_dq_kept" in kernels()
-    ops.set_keep_ds_max_bytes(0)
+    # opt-in: without a budget the backward recomputes (no dS scratch is taken behind the caller's back)
+    assert ops.keep_ds_max_bytes(dev) == 0
+    assert "attn_bwd_dq_pipe" in kernels()
+    assert "attn_bwd_dq_kept" in kernels(keep_ds=True)
+    ops.set_keep_ds_max_bytes(1 << 30)
     try:
+        assert "attn_bwd_dq_kept" in kernels()
+        ops.set_keep_ds_max_bytes(1 << 10)            # a budget below what this shape needs
         assert "attn_bwd_dq_pipe" in kernels()
-        assert "attn_bwd_dq_kept" in kernels(keep_ds=True)
     finally:
         ops.set_keep_ds_max_bytes(None)
+    # scratch that the arena already holds costs nothing more: used whatever the budget says
+    from odysseus_transformer_amd.utils import globals as g
+    g._set_global_memory_buffer(dev)
+    try:
+        assert "attn_bwd_dq_pipe" in kernels()
+        g.get_global_memory_buffer().get_tensor((4 << 20,), torch.uint8, "attn_bwd_workspace")
+        assert "attn_bwd_dq_kept" in kernels()
+    finally:
+        g._destroy_global_memory_buffer()
     with pytest.raises(ValueError):
         ops.attn_bwd(q[:, :500], k[:, :500], v[:, :500], o[:, :500], lse[:, :, :500].contiguous(), do[:, :500],
                      causal=True, keep_ds=True)

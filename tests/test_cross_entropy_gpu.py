@@ -85,3 +85,24 @@ def test_cross_entropy_training_shape(dev):
     _, _, _, dx_ref = oracle.cross_entropy_fwd_bwd(x.float(), y, grad_loss=loss_ref.item())
     assert abs(loss.item() - loss_ref.item()) <= 1e-5 * loss_ref.item()
     assert rel_err(logits.detach(), dx_ref) <= TOL_BF16
+
+
+def test_cross_entropy_label_out_of_range_is_loud(dev):
+    """A label outside [0, V) that is not ignore_index makes the loss NaN (never a token silently dropped); the mean
+    over zero counted tokens is 0 (the one documented deviation from 0 / 0)."""
+    from odysseus_transformer_amd.losses.cross_entropy import CrossEntropyLoss, cross_entropy_fwd
+    T, V = 16, 100
+    x = randn((T, V), 21).to(dev)
+    y = _labels(T, V, 22).to(dev)
+    bad = y.clone()
+    bad[3] = V          # off by one
+    losses, _, reduced = cross_entropy_fwd(x, bad)
+    assert torch.isnan(losses[3]) and not torch.isnan(losses[[0, 1, 2, 4]]).any()
+    assert torch.isnan(reduced[0]) and reduced[1].item() == T
+    xg = x.clone().requires_grad_(True)
+    loss = CrossEntropyLoss(reduction="sum")(xg, bad)
+    assert torch.isnan(loss)
+    bad[3] = -5
+    assert torch.isnan(CrossEntropyLoss()(x, bad))
+    none = torch.full((T,), -100, dtype=torch.int64, device=dev)
+    assert CrossEntropyLoss()(x, none).item() == 0.0

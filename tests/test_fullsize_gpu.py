@@ -19,6 +19,17 @@ from sampled import edge_samples, sampled_checks
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _kept_ds_budget():
+    """Kept dS is opt-in; these tests opt in (a quarter of the device's memory, as the benchmark does) so that the
+    full-size runs cover the kept-dS kernels.  The recomputing kernels are covered at full size by
+    test_fullsize_gpu.py::test_cfg2_shard_whole_result and at small sizes by test_attention_gpu.py."""
+    from odysseus_transformer_amd import ops
+    ops.set_keep_ds_max_bytes(torch.cuda.get_device_properties(0).total_memory // 4)
+    yield
+    ops.set_keep_ds_max_bytes(None)
+
+
 def run_attention(q, k, v, do, dev, causal=True, keep_ds=None):
     from odysseus_transformer_amd import ops
     qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))

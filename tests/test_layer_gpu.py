@@ -6,7 +6,7 @@ import zlib
 import pytest
 import torch
 
-from conftest import TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
+from conftest import assert_parity, TOL_BF16, TOL_F32, TOL_LSE, randn, rel_err
 import odysseus_oracle as oracle
 
 pytestmark = pytest.mark.gpu
@@ -69,14 +69,14 @@ def test_decoder_layer_fwd_bwd(case, dev):
     y = layer(xg, position_ids=pos)
     y.backward(dy.to(dev))
     torch.cuda.synchronize()
-    assert rel_err(y, y_ref) <= tol, "y"
+    assert_parity(y, y_ref, tol, f"{name} y")
     got = {
         "x": xg.grad, "ln1": layer.input_layernorm.weight.grad, "w_qkv": layer.self_attn.qkv_proj.weight.grad,
         "w_o": layer.self_attn.o_proj.weight.grad, "ln2": layer.post_attention_layernorm.weight.grad,
         "w_gate_up": layer.mlp.gate_up_proj.weight.grad, "w_down": layer.mlp.down_proj.weight.grad,
     }
     for k, v in got.items():
-        assert rel_err(v, g_ref[k]) <= tol, f"grad {k}: {rel_err(v, g_ref[k])}"
+        assert_parity(v, g_ref[k], tol, f"{name} grad {k}")
 
 
 def test_attention_block_unpacked_equals_packed(dev):
@@ -261,3 +261,62 @@ def test_linears_follow_autocast(dev):
         assert rel_err(m.weight.grad, x.detach().cpu()[0].sum(0)[None].expand(768, 512)) <= TOL_BF16
         with pytest.raises(TypeError):               # outside autocast a dtype mismatch still raises
             m(x.bfloat16())
+
+
+def test_fused_attention_under_inference_mode_and_with_hooks(dev):
+    """The fused projection -> rotary -> attention node must work on position ids created under
+    torch.inference_mode() (such tensors carry no version counter), and a forward hook registered on a projection
+    must still run: its presence sends the call down the module-by-module path, with the same result."""
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    d, H, Hkv, D, L = 512, 4, 2, 128, 320
+    attn = LlamaFlashAttention2TPSP(_config(d, H, Hkv, D, 1024), 0).to(torch.bfloat16).to(dev)
+    attn.fuse_rope = True
+    with torch.no_grad():
+        attn.qkv_proj.weight.copy_(randn(((H + 2 * Hkv) * D, d), 41, std=0.02))
+        attn.o_proj.weight.copy_(randn((d, H * D), 42, std=0.02))
+    x = randn((1, L, d), 43, dtype=torch.bfloat16).to(dev)
+    y_ref, _ = oracle.attention_block(x.float().cpu(), attn.qkv_proj.weight.float().cpu(), attn.o_proj.weight.float().cpu(),
+                                      H, Hkv, D)
+    with torch.inference_mode():
+        pos = torch.arange(L, device=dev)[None]
+        y1 = attn(x, position_ids=pos)[0]
+        y2 = attn(x, position_ids=pos)[0]            # second layer call with the same position tensor: the cached table
+    assert torch.equal(y1, y2)
+    assert rel_err(y1, y_ref) <= TOL_BF16
+    seen = []
+    handle = attn.qkv_proj.register_forward_hook(lambda mod, args, out: seen.append(tuple(out.shape)))
+    try:
+        y3 = attn(x, position_ids=torch.arange(L, device=dev)[None])[0]
+    finally:
+        handle.remove()
+    assert seen == [(1, L, (H + 2 * Hkv) * D)], "the hook on qkv_proj did not run"
+    assert rel_err(y3, y_ref) <= TOL_BF16 and rel_err(y3, y1.float()) <= 1e-2
+
+
+def test_zigzag_ring_patch_on_a_mistral_host(dev):
+    """apply_zigzag_ring_attn_patch_mistral (decoder/ring.py:107-113): a small transformers Mistral whose attention
+    goes through the HIP kernel gives the logits of the same model with the host's own eager attention in fp32."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import MistralConfig, MistralForCausalLM
+    from odysseus_transformer_amd.decoder.ring import apply_zigzag_ring_attn_patch_mistral, apply_zigzag_ring_attn_patch_llama
+    assert callable(apply_zigzag_ring_attn_patch_llama)
+    torch.manual_seed(0)
+    cfg = MistralConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+                        num_key_value_heads=1, head_dim=128, vocab_size=128, max_position_embeddings=2048,
+                        sliding_window=None, rms_norm_eps=1e-6)
+    cfg._attn_implementation = "eager"
+    host = MistralForCausalLM(cfg)
+    L = 300
+    ids = torch.randint(0, 128, (1, L), generator=torch.Generator().manual_seed(2))
+    pos = torch.arange(L)[None]
+    with torch.no_grad():
+        ref = host(ids, position_ids=pos, use_cache=False).logits.float()
+    model = MistralForCausalLM(cfg)
+    model.load_state_dict(host.state_dict())
+    model = model.to(torch.bfloat16).to(dev)
+    apply_zigzag_ring_attn_patch_mistral(model)
+    assert model.config._attn_implementation == "flash_attention_2"
+    with torch.no_grad():
+        logits = model(ids.to(dev), position_ids=pos.to(dev), use_cache=False).logits
+    # bf16 weights and activations against the fp32 host: the bar of a whole bf16 model, not of one kernel
+    assert rel_err(logits, ref) <= 5e-2

@@ -10,6 +10,17 @@ import odysseus_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _kept_ds_budget():
+    """Kept dS is opt-in; these tests opt in (a quarter of the device's memory, as the benchmark does) so that the
+    full-size runs cover the kept-dS kernels.  The recomputing kernels are covered at full size by
+    test_fullsize_gpu.py::test_cfg2_shard_whole_result and at small sizes by test_attention_gpu.py."""
+    from odysseus_transformer_amd import ops
+    ops.set_keep_ds_max_bytes(torch.cuda.get_device_properties(0).total_memory // 4)
+    yield
+    ops.set_keep_ds_max_bytes(None)
+
+
 def _local(t, rank, world, dim=1):
     """Chunks r and 2N-1-r of the sequence (utils/apply_seq_parallel.py:93-99)."""
     ch = t.chunk(2 * world, dim=dim)
