@@ -61,13 +61,14 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
   ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_fwd: scale must be positive");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == ODY_BF16 && D == 128) {
-    const size_t need = ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype);
+    // the least that will do: without room for the parts of a key-split call the call runs unsplit
+    const size_t need = (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255;
     ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_fwd: workspace is NULL");
     ODY_REQUIRE(workspace_bytes >= need, ODY_ERR_WORKSPACE, "ody_attn_fwd: workspace of %zu bytes, %zu needed",
                 workspace_bytes, need);
     ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
                 "ody_attn_fwd: workspace must be 256-byte aligned");
-    return ody_launch_attn_fwd_w8(p, workspace, st);
+    return ody_launch_attn_fwd_w8(p, workspace, workspace_bytes, st);
   }
   if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
   return ody_launch_attn_fwd_f32(p, D, st);
@@ -106,7 +107,9 @@ extern "C" int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v,
                                     float scale, int causal, int dtype, void* stream) {
   int rc = check_common("ody_attn_fwd_noalloc", B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
-  const size_t need = ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, dtype);
+  // the fixed scratch holds the flags and the V images; a call that would cut its key range runs unsplit here
+  const size_t need = (dtype == ODY_BF16 && D == 128)
+                          ? ((ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255) : 0;
   ODY_REQUIRE(need <= (size_t)ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES, ODY_ERR_WORKSPACE,
               "ody_attn_fwd_noalloc: this shape needs %zu bytes of scratch, the library-owned buffer holds %zu "
               "(256 bytes per key row of every kv head: B*Hkv*Lk <= about 131000); use ody_attn_fwd with a "
@@ -119,7 +122,7 @@ extern "C" int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v,
 
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype) {
   if (B <= 0 || Lq <= 0 || Lk <= 0 || Hq <= 0 || Hkv <= 0) return 0;
-  if (dtype == ODY_BF16 && D == 128) return (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv) + 255) & ~(size_t)255;
+  if (dtype == ODY_BF16 && D == 128) return (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, true) + 255) & ~(size_t)255;
   return 0;
 }
 

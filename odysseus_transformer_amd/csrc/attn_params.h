@@ -45,10 +45,11 @@ struct AttnParams {
 // walk the same K / V (or Q / dO) tiles at the same time, sharing them through its L2.
 struct BlockCoord { int rank, h, b; };
 #ifdef __HIPCC__
-__device__ __forceinline__ BlockCoord ody_block_coord(int H, int B) {
-  const int id = blockIdx.x, hb = id % (H * B);
+__device__ __forceinline__ BlockCoord ody_block_coord_of(int id, int H, int B) {
+  const int hb = id % (H * B);
   return BlockCoord{id / (H * B), hb % H, hb / H};
 }
+__device__ __forceinline__ BlockCoord ody_block_coord(int H, int B) { return ody_block_coord_of(blockIdx.x, H, B); }
 #endif
 
 // Launchers (one per translation unit); each returns an ody_status.
@@ -61,9 +62,11 @@ int ody_launch_attn_images(const void* src, const AttnStrides& s, int B, int L, 
 // head_dim 128 backward, everything that depends on the queries only, in one launch: p.delta, the transposed images
 // of Q and dO and the start values (1 KB per 64-query tile)
 int ody_launch_attn_bwd_prepass(const AttnParams& p, void* qimg, void* doimg, void* stats, hipStream_t st);
-// head_dim 128 only, 8 wavefronts x 32 queries per block; workspace of ody_attn_fwd_w8_workspace(...) bytes
-int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, hipStream_t st);
-size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv);
+// head_dim 128 only, 8 wavefronts x 32 queries per block; workspace of ody_attn_fwd_w8_workspace(...) bytes.
+// with_split: with room for the fp32 parts of a call whose fully visible key range is cut into 2 or 4 parts (few query
+// blocks against many keys); a workspace without that room makes such a call run unsplit.
+int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, size_t workspace_bytes, hipStream_t st);
+size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv, bool with_split);
 // the online-rescaling forward kernel restricted to query blocks of `block` rows whose flag is set
 int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st);
 // head_dim 128 only; workspace of ody_attn_bwd_pipe_workspace(...) bytes (p.delta is set separately)

@@ -318,3 +318,45 @@ def test_attention_bwd_kept_ds_full_blocks(case, dev):
     dq2, dk2, dv2 = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=False, keep_ds=False)
     assert torch.equal(dk2, dk) and torch.equal(dv2, dv)
     assert_parity(dq2, dq_ref, TOL_BF16, "dq of the recomputing kernel", 1e-3)
+
+
+@pytest.mark.parametrize("case", [(1, 512, 4096, 2, 2, 4), (1, 300, 2100, 4, 1, 2), (2, 256, 1100, 2, 2, 2), (1, 2048, 1024, 4, 4, 2)],
+                         ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_parts%d" % c)
+def test_attention_fwd_key_split(case, dev):
+    """Few query blocks against many fully visible keys (the off-diagonal steps of a ring): the forward cuts the key
+    range into parts, one block per (query block, part), and merges them.  Same (out, lse) as the oracle, the
+    overflow fallback still reaches the blocks it must, and a workspace without room for the parts (the
+    allocation-free entry point's) gives the unsplit result."""
+    from odysseus_transformer_amd import ops, _lib
+    B, Lq, Lk, Hq, Hkv, parts = case
+    D = 128
+    print(f"key split case={case}", flush=True)
+    lib = _lib.load()
+    with_parts = lib.ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _lib.ODY_BF16)
+    per_part = ((B * Lq * Hq * D * 4 + 255) & ~255) + ((B * Hq * Lq * 4 + 255) & ~255)
+    flags_and_images = ((B * Hq * ((Lq + 255) // 256) * 4 + 255) & ~255) + B * Hkv * ((Lk + 63) // 64) * 16384
+    assert with_parts >= flags_and_images + parts * (per_part - 512), "the workspace query leaves no room for the parts"
+    q, k, v, _ = _inputs(B, Lq, Lk, Hq, Hkv, D, torch.bfloat16, seed=23)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=False)
+    qg, kg, vg = (t.to(dev) for t in (q, k, v))
+    _lib.profile_enable(True)
+    try:
+        o, lse = ops.attn_fwd(qg, kg, vg, causal=False)
+        torch.cuda.synchronize()
+        assert "attn_fwd_split_merge" in _lib.profile_collect()
+    finally:
+        _lib.profile_enable(False)
+    assert_parity(o, o_ref, TOL_BF16, "o")
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
+    # unsplit through the allocation-free entry point: the same numbers up to the rounding of the merge
+    o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
+    ops.attn_fwd_noalloc(qg, kg, vg, o2, lse2, causal=False)
+    assert_parity(o2, o_ref, TOL_BF16, "o unsplit")
+    assert rel_err(o, o2.float()) <= 1e-2 and torch.allclose(lse, lse2, atol=1e-4, rtol=1e-4)
+    # late keys far above the early ones: the parts' references differ, and the blocks that overflow are redone
+    q[:, :, 0], k[:, :, 0] = 2.0, -4.0
+    k[:, Lk // 2 + 40:Lk // 2 + 60, 0] = 4.0
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=False)
+    o, lse = ops.attn_fwd(q.to(dev), k.to(dev), vg, causal=False)
+    assert_parity(o, o_ref, TOL_BF16, "o with late large scores")
+    assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
