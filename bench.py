@@ -163,7 +163,9 @@ def mfma_sustained(_lib, dev):
                 e1.record()
                 torch.cuda.synchronize()
                 best = e0.elapsed_time(e1) if best is None else min(best, e0.elapsed_time(e1))
-            res[name + tag + "_tflops"] = round(blocks * 4 * iters * 16 * 32768.0 / (best * 1e-3) / 1e12, 1)
+            # per iteration and wavefront: 16 MFMAs of 32768 FLOP, or 64 of 16384 (the 128 x 128 tile with k = 32)
+            flop = blocks * 4 * iters * (16 * 32768.0 if shape == 0 else 64 * 16384.0)
+            res[name + tag + "_tflops"] = round(flop / (best * 1e-3) / 1e12, 1)
     return res
 
 

@@ -38,8 +38,8 @@ __device__ __forceinline__ float ody_exp2(float x) { return __builtin_amdgcn_exp
 // ---------------------------------------------------------------------------
 // MFMA-only loops on register operands: the sustained rate of the matrix pipe for given operand data, with
 // either bf16 instruction shape.  shape 0: v_mfma_f32_32x32x16_bf16, 16 accumulator tiles (a 128 x 128 wavefront
-// tile); shape 1: v_mfma_f32_16x16x32_bf16, 64 accumulator tiles (the same tile and operand reuse).  4 wavefronts
-// per block; FLOP = blocks * 4 * iters * 16 * 32768 either way.
+// tile, k = 16 per iteration); shape 1: v_mfma_f32_16x16x32_bf16, 64 accumulator tiles (the same tile, k = 32 per
+// iteration).  4 wavefronts per block; FLOP = blocks * 4 * iters * 16 * 32768 for shape 0, twice that for shape 1.
 // ---------------------------------------------------------------------------
 namespace {
 template <int SHAPE>
