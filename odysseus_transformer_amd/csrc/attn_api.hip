@@ -107,9 +107,14 @@ extern "C" int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v,
                                     float scale, int causal, int dtype, void* stream) {
   int rc = check_common("ody_attn_fwd_noalloc", B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
-  // the fixed scratch holds the flags and the V images; a call that would cut its key range runs unsplit here
-  const size_t need = (dtype == ODY_BF16 && D == 128)
-                          ? ((ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255) : 0;
+  // the fixed scratch holds the flags and the V images, and the parts of a call that cuts its key ranges if they fit
+  // as well (then the result is that of ody_attn_fwd bit for bit); otherwise such a call runs unsplit here
+  size_t need = 0;
+  if (dtype == ODY_BF16 && D == 128) {
+    need = (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, true) + 255) & ~(size_t)255;
+    if (need > (size_t)ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES)
+      need = (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255;
+  }
   ODY_REQUIRE(need <= (size_t)ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES, ODY_ERR_WORKSPACE,
               "ody_attn_fwd_noalloc: this shape needs %zu bytes of scratch, the library-owned buffer holds %zu "
               "(256 bytes per key row of every kv head: B*Hkv*Lk <= about 131000); use ody_attn_fwd with a "

@@ -12,10 +12,10 @@
 // outgrows the reference by more than fp32 can hold shows up as a row sum that overflowed; the
 // 256-query block is then flagged and redone by the online-rescaling kernel.
 //
-// A step with few queries against many keys (the off-diagonal steps of a ring: 8192 queries are 32 query blocks per
-// head) leaves compute units idle: then the fully visible key range is cut into 2 or 4 parts, one block per
-// (query block, part); each writes its normalised partial result and log-sum-exp in fp32 and a small kernel merges
-// the parts with the arithmetic of the ring's block merge.
+// A call with few query blocks (16384 queries are 64 per head; the off-diagonal steps of a zigzag ring have 32) leaves
+// compute units idle or, under a causal mask, waiting for the one with the longest block: then every block's key range
+// is cut into 2 or 4 parts, one block per (query block, part); each writes its normalised partial result and
+// log-sum-exp in fp32 and a small kernel merges the parts with the arithmetic of the ring's block merge.
 #include "attn_params.h"
 #include "attn_tile.h"
 
@@ -29,8 +29,10 @@ constexpr int FW_STAGE = TILE_ELEMS + IMG_ELEMS;   // K tile, V^T image
 static_assert(FW_WAVES == 8, "the load split and the vmcnt waits assume 8 wavefronts");
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
-// nsplit > 1 (fully visible keys only): block id = split + nsplit * (the usual id); part_out [split][B][Lq][Hq][D] and
-// part_lse [split][B][Hq][Lq] in fp32 take the place of p.out / p.lse.
+// nsplit > 1: block id = split + nsplit * (the usual id), the block takes part `split` of its tiles; part_out
+// [split][B][Lq][Hq][D] and part_lse [split][B][Hq][Lq] in fp32 take the place of p.out / p.lse.  Under a causal mask a
+// later part may start beyond the first keys of some of its queries: their reference is then 0 instead of a score,
+// which the overflow flag covers like any other reference that turns out too low.
 __global__ __launch_bounds__(FW_THREADS) void attn_fwd_w8_kernel(const AttnParams p, const bf16* __restrict__ vimg,
                                                                   int* __restrict__ bail_flags, int nsplit,
                                                                   float* __restrict__ part_out,
@@ -262,12 +264,16 @@ __global__ __launch_bounds__(256) void attn_fwd_split_merge_kernel(const AttnPar
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
-// Parts of the key range for a call with fully visible keys: as many as it takes to give every compute unit of an
-// MI355X (256) a block, at most 4, and none for a key range of fewer than 8 tiles per part.
-int key_splits(int B, int Lq, int Lk, int Hq) {
+// Parts of a query block's key range.  With fewer blocks than it takes to keep the chip's 256 compute units busy and
+// balanced -- one block each when all blocks are equally long (fully visible keys), two each when they are not (under
+// a causal mask block i is i + 1 tiles long, and only with a second, lighter block per unit does the heaviest-first
+// order even that out) -- the range is cut into 2 or 4 parts of at least 8 tiles (on average, when causal).
+int key_splits(int B, int Lq, int Lk, int Hq, bool causal) {
   const int64_t blocks = (int64_t)B * Hq * ((Lq + FW_BM - 1) / FW_BM);
+  const int64_t want = causal ? 512 : 256;
+  const int tiles = ((causal ? min(Lk, Lq + max(Lk - Lq, 0)) : Lk) + BN - 1) / BN;
   int s = 1;
-  while (s < 4 && blocks * s * 2 <= 256 && (Lk + BN - 1) / BN >= 16 * s) s *= 2;
+  while (s < 4 && blocks * s * 2 <= want && tiles >= 16 * s) s *= 2;
   return s;
 }
 
@@ -277,7 +283,7 @@ int key_splits(int B, int Lq, int Lk, int Hq) {
 size_t ody_attn_fwd_w8_workspace(int B, int Lq, int Lk, int Hq, int Hkv, bool with_split) {
   const size_t flags = align256((size_t)B * Hq * ((Lq + FW_BM - 1) / FW_BM) * sizeof(int));
   size_t n = flags + align256(ody_attn_images_bytes(B, Lk, Hkv));
-  const int ns = with_split ? key_splits(B, Lq, Lk, Hq) : 1;
+  const int ns = with_split ? max(key_splits(B, Lq, Lk, Hq, false), key_splits(B, Lq, Lk, Hq, true)) : 1;
   if (ns > 1) n += align256((size_t)ns * B * Lq * Hq * D * sizeof(float)) + align256((size_t)ns * B * Hq * Lq * sizeof(float));
   return n;
 }
@@ -293,9 +299,9 @@ int ody_launch_attn_fwd_w8(const AttnParams& p, void* workspace, size_t workspac
   bf16* images = reinterpret_cast<bf16*>(w + align256((size_t)nflags * sizeof(int)));
   rc = ody_launch_attn_images(p.v, p.sv, p.B, p.Lk, p.Hkv, images, flags, nflags, st);
   if (rc) return rc;
-  // the key split: fully visible keys only, and only where the caller's workspace has room for the parts (the
-  // allocation-free entry point's fixed scratch has not)
-  int ns = p.causal ? 1 : key_splits(p.B, p.Lq, p.Lk, p.Hq);
+  // the key split, where the caller's workspace has room for the parts (the allocation-free entry point's fixed
+  // scratch may not)
+  int ns = key_splits(p.B, p.Lq, p.Lk, p.Hq, p.causal != 0);
   if (ns > 1 && workspace_bytes < ody_attn_fwd_w8_workspace(p.B, p.Lq, p.Lk, p.Hq, p.Hkv, true)) ns = 1;
   float* part_out = nullptr;
   float* part_lse = nullptr;

@@ -320,43 +320,54 @@ def test_attention_bwd_kept_ds_full_blocks(case, dev):
     assert_parity(dq2, dq_ref, TOL_BF16, "dq of the recomputing kernel", 1e-3)
 
 
-@pytest.mark.parametrize("case", [(1, 512, 4096, 2, 2, 4), (1, 300, 2100, 4, 1, 2), (2, 256, 1100, 2, 2, 2), (1, 2048, 1024, 4, 4, 2)],
-                         ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_parts%d" % c)
+@pytest.mark.parametrize("case", [(1, 512, 4096, 2, 2, 4, False), (1, 300, 2100, 4, 1, 4, False), (2, 256, 1100, 2, 2, 2, False),
+                                  (1, 2048, 1024, 4, 4, 2, False), (1, 2048, 2048, 4, 4, 4, True), (1, 1100, 1500, 2, 1, 2, True)],
+                         ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_parts%d_c%d" % c)
 def test_attention_fwd_key_split(case, dev):
-    """Few query blocks against many fully visible keys (the off-diagonal steps of a ring): the forward cuts the key
-    range into parts, one block per (query block, part), and merges them.  Same (out, lse) as the oracle, the
-    overflow fallback still reaches the blocks it must, and a workspace without room for the parts (the
-    allocation-free entry point's) gives the unsplit result."""
+    """Few query blocks (the steps of a ring over 16384-token chunks): the forward cuts every block's key range into
+    parts, one block per (query block, part), and merges them.  Same (out, lse) as the oracle, the overflow fallback
+    still reaches the blocks it must, and a workspace without room for the parts gives the unsplit result."""
     from odysseus_transformer_amd import ops, _lib
-    B, Lq, Lk, Hq, Hkv, parts = case
+    B, Lq, Lk, Hq, Hkv, parts, causal = case
     D = 128
     print(f"key split case={case}", flush=True)
     lib = _lib.load()
     with_parts = lib.ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _lib.ODY_BF16)
     per_part = ((B * Lq * Hq * D * 4 + 255) & ~255) + ((B * Hq * Lq * 4 + 255) & ~255)
-    flags_and_images = ((B * Hq * ((Lq + 255) // 256) * 4 + 255) & ~255) + B * Hkv * ((Lk + 63) // 64) * 16384
-    assert with_parts >= flags_and_images + parts * (per_part - 512), "the workspace query leaves no room for the parts"
+    unsplit = ((B * Hq * ((Lq + 255) // 256) * 4 + 255) & ~255) + B * Hkv * ((Lk + 63) // 64) * 16384
+    assert with_parts >= unsplit + parts * (per_part - 512), "the workspace query leaves no room for the parts"
     q, k, v, _ = _inputs(B, Lq, Lk, Hq, Hkv, D, torch.bfloat16, seed=23)
-    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=False)
+
+    def unsplit_fwd(qg, kg, vg):
+        """through the C ABI with a workspace that has room for the flags and the V images only"""
+        out = torch.empty_like(qg)
+        lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=dev)
+        ws = torch.empty(unsplit, dtype=torch.uint8, device=dev)
+        _lib.call("ody_attn_fwd", qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), out.data_ptr(), lse.data_ptr(), B, Lq, Lk, Hq,
+                  Hkv, D, *ops._blhd(qg, "q"), *ops._blhd(kg, "k"), *ops._blhd(vg, "v"), *ops._blhd(out, "out"),
+                  1.0 / math.sqrt(D), int(causal), _lib.ODY_BF16, ws.data_ptr(), unsplit, torch.cuda.current_stream().cuda_stream)
+        return out, lse
+
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal)
     qg, kg, vg = (t.to(dev) for t in (q, k, v))
     _lib.profile_enable(True)
     try:
-        o, lse = ops.attn_fwd(qg, kg, vg, causal=False)
+        o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
         torch.cuda.synchronize()
         assert "attn_fwd_split_merge" in _lib.profile_collect()
+        o2, lse2 = unsplit_fwd(qg, kg, vg)
+        torch.cuda.synchronize()
+        assert "attn_fwd_split_merge" not in _lib.profile_collect()
     finally:
         _lib.profile_enable(False)
     assert_parity(o, o_ref, TOL_BF16, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
-    # unsplit through the allocation-free entry point: the same numbers up to the rounding of the merge
-    o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
-    ops.attn_fwd_noalloc(qg, kg, vg, o2, lse2, causal=False)
     assert_parity(o2, o_ref, TOL_BF16, "o unsplit")
     assert rel_err(o, o2.float()) <= 1e-2 and torch.allclose(lse, lse2, atol=1e-4, rtol=1e-4)
     # late keys far above the early ones: the parts' references differ, and the blocks that overflow are redone
     q[:, :, 0], k[:, :, 0] = 2.0, -4.0
     k[:, Lk // 2 + 40:Lk // 2 + 60, 0] = 4.0
-    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=False)
-    o, lse = ops.attn_fwd(q.to(dev), k.to(dev), vg, causal=False)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal)
+    o, lse = ops.attn_fwd(q.to(dev), k.to(dev), vg, causal=causal)
     assert_parity(o, o_ref, TOL_BF16, "o with late large scores")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
