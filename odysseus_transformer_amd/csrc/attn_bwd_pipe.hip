@@ -14,6 +14,7 @@
 //      dQ^T += K^T dS^T       A: K^T image (LDS)     B: dS^T = accumulator layout
 //
 // dK/dV kernel -- key-stationary, 32 keys per wavefront (described where it is defined).
+#include <algorithm>
 #include <type_traits>
 #include <utility>
 #include "attn_params.h"
@@ -302,9 +303,10 @@ __host__ __device__ inline int64_t ds_block_index(int nbq, int kb, int qb, bool 
 // (beyond Lq, or a query that saw no key) hold -1e30.
 //
 // SPLIT = false: a block owns 256 keys of one kv head and walks all query heads of its group.
-// SPLIT = true (grouped-query attention): a block owns 256 keys for ONE query head and writes
-// fp32 partial dK / dV to `part`, which attn_bwd_group_sum_kernel adds up over the group.  With few
-// kv heads this is what gives the chip enough, and evenly sized, blocks.
+// SPLIT = true (grouped-query attention, or too few key blocks for the chip): a block owns 256 keys for ONE query
+// head and part `bc.h % qparts` of that head's query tiles, and writes fp32 partial dK / dV to `part`, which
+// attn_bwd_group_sum_kernel adds up over the group and the parts.  With few kv heads, or few keys against many
+// queries (a ring step over a short key block), this is what gives the chip enough, and evenly sized, blocks.
 //
 // KEEP_DS = true (whole 256-row blocks on both sides; causal: self-attention): every dS tile also goes to p.ds, in the
 // layout described at ds_block_index, and the dQ kernel below (attn_bwd_dq_kept_kernel) reads it back
@@ -314,15 +316,16 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
                                                                          const bf16* __restrict__ qimg,
                                                                          const bf16* __restrict__ doimg,
                                                                          const bf16* __restrict__ stats,
-                                                                         float* __restrict__ part) {
+                                                                         float* __restrict__ part, int qparts) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* ring = reinterpret_cast<bf16*>(smem_raw);   // [2][KV_STAGE]
 
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
             i = lane & 31;
-  const BlockCoord bc = ody_block_coord(SPLIT ? p.Hq : p.Hkv, p.B);   // rank 0 = first key block = most query tiles
-  const int hk = SPLIT ? bc.h / p.group : bc.h, b = bc.b;
-  const int h_first = SPLIT ? bc.h : hk * p.group, n_heads = SPLIT ? 1 : p.group;   // query heads this block walks
+  const BlockCoord bc = ody_block_coord(SPLIT ? p.Hq * qparts : p.Hkv, p.B);   // rank 0 = first key block = most query tiles
+  const int hq = SPLIT ? bc.h / qparts : 0, qpart = SPLIT ? bc.h % qparts : 0;
+  const int hk = SPLIT ? hq / p.group : bc.h, b = bc.b;
+  const int h_first = SPLIT ? hq : hk * p.group, n_heads = SPLIT ? 1 : p.group;   // query heads this block walks
   const int n0 = bc.rank * KV_BN, wn0 = n0 + wave * 32, key = wn0 + i;
   const int q_tiles = (p.Lq + KV_BQ - 1) / KV_BQ;
   simd_stagger(tid);
@@ -349,14 +352,19 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
     for (int r = 0; r < 16; r++) dk[dt][r] = dv[dt][r] = 0.f;
 
   const int t_begin = p.causal ? max(0, n0 - p.off) / KV_BQ : 0;   // first query tile that sees a key of this block
-  const int ntq = max(0, q_tiles - t_begin);
+  int ntq = max(0, q_tiles - t_begin), t_top = q_tiles - 1;   // this block's tiles: t_top, t_top - 1, ... (ntq of them)
+  if (SPLIT && qparts > 1) {
+    const int per = (ntq + qparts - 1) / qparts;
+    t_top -= qpart * per;
+    ntq = max(0, min(per, ntq - qpart * per));
+  }
   const int total = ntq * n_heads;   // flattened (query head, query tile)
   const float c2 = p.scale_log2e;
 
   // Direct loads of one stage: uniform base pointers plus 32-bit per-lane offsets that are
   // recomputed from the lane id every time (cheaper than keeping them in registers here).
   auto load_stage = [&](bf16* st, int it, int j) {   // j = 0, 1: the two halves of the stage's loads
-    const int hg = it / ntq, t = q_tiles - 1 - (it % ntq), h = h_first + hg;
+    const int hg = it / ntq, t = t_top - (it % ntq), h = h_first + hg;
     const bf16* qp = static_cast<const bf16*>(p.q) + b * p.sq.b + h * p.sq.h + (int64_t)t * KV_BQ * p.sq.l;
     const bf16* dop = static_cast<const bf16*>(p.dout) + b * p.sdo.b + h * p.sdo.h + (int64_t)t * KV_BQ * p.sdo.l;
     const int64_t tile_id = ((int64_t)b * p.Hq + h) * q_tiles + t;
@@ -470,7 +478,7 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
   for (int it = 0; it < total; it++) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    const int t = q_tiles - 1 - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
+    const int t = t_top - (it % ntq);   // last query tile first: the key blocks of an XCD then read the same
                                               // Q / dO tiles at the same time and share them through L2
     const bf16* st = ring + (it & 1) * KV_STAGE;
     // every query of the tile is before every key of this wavefront: nothing to do
@@ -494,9 +502,9 @@ __global__ __launch_bounds__(KV_THREADS) void attn_bwd_dkdv_pipe_kernel(const At
 
   if (SPLIT) {
     if (key < p.Lk) {
-      // part: [dK | dV][batch][query head][key][D] fp32, unscaled
-      float* pk = part + (((int64_t)b * p.Hq + h_first) * p.Lk + key) * D;
-      float* pv = pk + (int64_t)p.B * p.Hq * p.Lk * D;
+      // part: [dK | dV][batch][query head][part of the queries][key][D] fp32, unscaled
+      float* pk = part + (((int64_t)b * p.Hq * qparts + bc.h) * p.Lk + key) * D;
+      float* pv = pk + (int64_t)p.B * p.Hq * qparts * p.Lk * D;
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -579,7 +587,12 @@ constexpr int DS_PIECE_ELEMS = GROUP_ELEMS;   // 1 KB + 16 bytes: consecutive pi
 constexpr int DQK_DS_BUF = 32 * DS_PIECE_ELEMS, DQK_SETS = 4;
 constexpr int DQK_LDS_ELEMS = 2 * DQK_DS_BUF + 2 * IMG_ELEMS;
 
-__global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const AttnParams p, const bf16* __restrict__ kimg) {
+//
+// kparts > 1 (too few query blocks for the chip: a ring step of few queries against a long key block): block id =
+// part + kparts * (the usual id), the block takes part `part` of its 256-key blocks and leaves its unscaled fp32 sum in
+// dq_part [part][B][Lq][Hq][D]; attn_bwd_dq_sum_kernel adds the parts and finishes dq.
+__global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const AttnParams p, const bf16* __restrict__ kimg,
+                                                                       int kparts, float* __restrict__ dq_part) {
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* dsbuf = reinterpret_cast<bf16*>(smem_raw);   // [2][DQK_DS_BUF]
@@ -587,16 +600,37 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
 
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
             i = lane & 31;
-  const BlockCoord bc = ody_block_coord(p.Hq, p.B);
-  const int nqb = gridDim.x / (p.Hq * p.B);
+  const int kpart = blockIdx.x % kparts;
+  const BlockCoord bc = ody_block_coord_of(blockIdx.x / kparts, p.Hq, p.B);
+  const int nqb = gridDim.x / (p.Hq * p.B * kparts);
   const int qblk = p.causal ? nqb - 1 - bc.rank : bc.rank;   // causal: heaviest blocks first
   const int h = bc.h, b = bc.b, hk = h / p.group;
   const int x = wave >> 1, mt = wave & 1, nbq = p.Lq / KV_BN, nbk = p.Lk / KV_BN;
   const bf16* kip = kimg + ((int64_t)b * p.Hkv + hk) * (p.Lk / 64) * IMG_ELEMS;
   const bf16* dsh = p.ds + ((int64_t)b * p.Hq + h) * ds_blocks_per_head(nbq, nbk, p.causal) * DS_BLOCK_ELEMS;
   // 64-key tiles: all of them, or (causal) those up to the block's last query; a multiple of DQK_SETS
-  const int ntiles = p.causal ? 4 * (qblk + 1) : 4 * nbk;
+  int ntiles = p.causal ? 4 * (qblk + 1) : 4 * nbk;
   const int last_tile = p.causal ? 4 * qblk + x : ntiles;   // of this wavefront's queries
+  int t_first = 0;   // this block's part of the tiles: [t_first, ntiles), whole 256-key blocks
+  if (kparts > 1) {
+    const int per = 4 * ((ntiles / 4 + kparts - 1) / kparts);
+    t_first = min(kpart * per, ntiles);
+    ntiles = min(t_first + per, ntiles);
+  }
+  // position 32 mt + i of the tile's kept order = chunk 4 mt + (i >> 3), element i & 7
+  const int qrow = qblk * DQ_BM + KV_BQ * x + 32 * ((i >> 2) & 1) + 16 * ((i >> 3) & 1) + 4 * (i & 3) + (i >> 4) + 2 * mt;
+  auto store_part = [&](const f32x16 (&acc)[DT]) {
+    float* dst = dq_part + ((((int64_t)kpart * p.B + b) * p.Lq + qrow) * p.Hq + h) * D;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int a = 0; a < 4; a++) {
+        f32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = acc[dt][4 * a + e];
+        *reinterpret_cast<f32x4*>(dst + 32 * dt + 8 * a + 4 * g) = w;
+      }
+  };
 
   u32x4 regs[DQK_SETS][6];
   // tile t: this wavefront's 4 of the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk) -- 32 KB in a row --
@@ -624,14 +658,17 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
     for (int j = 0; j < 2; j++)
       *reinterpret_cast<u32x4*>(slot + ((DQ_WAVES * j + wave) * 64 + lane) * 8) = regs[set][4 + j];
   };
-#pragma unroll
-  for (int u = 0; u < DQK_SETS; u++) issue(u, u);   // ntiles >= DQK_SETS
-
   f32x16 dq[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
 #pragma unroll
     for (int r = 0; r < 16; r++) dq[dt][r] = 0.f;
+  if (t_first >= ntiles) {   // a part without keys (causal: an early query block has fewer key blocks than parts)
+    store_part(dq);
+    return;
+  }
+#pragma unroll
+  for (int u = 0; u < DQK_SETS; u++) issue(u, t_first + u);   // ntiles - t_first >= DQK_SETS
 
   const int ibase = image_frag_base(g, i);
   // the transposing read: inside 16 lanes, lane 4 k + m supplies key 4 k (+ the fragment's row offset) and queries
@@ -664,9 +701,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
     }
   };
 
-  drain(0, 0);
+  drain(0, t_first);
   ISSUE_ORDER();
-  int t0 = 0;
+  int t0 = t_first;
   do {   // not a `for`: its entry test would give the compiler a block to sink the loads above into, out of order
 #pragma unroll
     for (int u = 0; u < DQK_SETS; u++) {
@@ -686,14 +723,68 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
     }
   } while ((t0 += DQK_SETS) < ntiles);
 
-  // position 32 mt + i of the tile's kept order = chunk 4 mt + (i >> 3), element i & 7
-  const int row = 32 * ((i >> 2) & 1) + 16 * ((i >> 3) & 1) + 4 * (i & 3) + (i >> 4) + 2 * mt;
-  store_dq_row(p, dq, b, h, qblk * DQ_BM + KV_BQ * x + row, g);
+  if (kparts > 1) store_part(dq);
+  else store_dq_row(p, dq, b, h, qrow, g);
 }
 
-// dK, dV of a kv head = sum of the fp32 partials of its query heads; one thread per 4 elements d..d+3 of the first half
-// of a key row and their partners d + 64 (the pairs of the rotary embedding)
-__global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParams p, const float* __restrict__ part) {
+// dq = the sum of the fp32 parts of a key-split attn_bwd_dq_kept_kernel, finished like store_dq_row does; one thread per
+// 4 elements d..d+3 of the first half of a (query, head) row and their partners d + 64 (the pairs of the rotary
+// embedding)
+__global__ __launch_bounds__(256) void attn_bwd_dq_sum_kernel(const AttnParams p, const float* __restrict__ dq_part, int kparts) {
+  constexpr int Q = D / 8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;   // over B * Lq * Hq * D / 8
+  const int64_t total = (int64_t)p.B * p.Lq * p.Hq * Q;
+  if (idx >= total) return;
+  const int d4 = idx % Q;
+  const int h = (idx / Q) % p.Hq;
+  const int qi = (idx / ((int64_t)Q * p.Hq)) % p.Lq;
+  const int b = idx / ((int64_t)Q * p.Hq * p.Lq);
+  const int64_t plane = (int64_t)p.B * p.Lq * p.Hq * D;
+  const float* src = dq_part + (((int64_t)b * p.Lq + qi) * p.Hq + h) * D + 4 * d4;
+  f32x4 s1 = {0.f, 0.f, 0.f, 0.f}, s2 = s1;
+  for (int s = 0; s < kparts; s++) {
+    s1 += *reinterpret_cast<const f32x4*>(src + s * plane);
+    s2 += *reinterpret_cast<const f32x4*>(src + s * plane + D / 2);
+  }
+  s1 *= p.scale;
+  s2 *= p.scale;
+  if (p.dq_f32) {
+    float* dqp = static_cast<float*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l + 4 * d4;
+    if (p.accumulate_dq) {
+      s1 += *reinterpret_cast<const f32x4*>(dqp);
+      s2 += *reinterpret_cast<const f32x4*>(dqp + D / 2);
+    }
+    *reinterpret_cast<f32x4*>(dqp) = s1;
+    *reinterpret_cast<f32x4*>(dqp + D / 2) = s2;
+    return;
+  }
+  bf16* dqp = static_cast<bf16*>(p.dq) + b * p.sdq.b + h * p.sdq.h + (int64_t)qi * p.sdq.l + 4 * d4;
+  bf16x4 w1, w2;
+  if (p.rope_q) {
+    const bf16x8 cs = *reinterpret_cast<const bf16x8*>(p.rope_q + ((int64_t)b * p.Lq + qi) * D + 8 * d4);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
+      w1[e] = (bf16)(s1[e] * c + s2[e] * sn);
+      w2[e] = (bf16)(s2[e] * c - s1[e] * sn);
+    }
+  } else {
+    if (p.accumulate_dq) {
+      const bf16x4 o1 = *reinterpret_cast<const bf16x4*>(dqp), o2 = *reinterpret_cast<const bf16x4*>(dqp + D / 2);
+#pragma unroll
+      for (int e = 0; e < 4; e++) s1[e] += (float)o1[e], s2[e] += (float)o2[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) w1[e] = (bf16)s1[e], w2[e] = (bf16)s2[e];
+  }
+  *reinterpret_cast<bf16x4*>(dqp) = w1;
+  *reinterpret_cast<bf16x4*>(dqp + D / 2) = w2;
+}
+
+// dK, dV of a kv head = sum of the fp32 partials of its query heads and their `qparts` parts; one thread per 4 elements
+// d..d+3 of the first half of a key row and their partners d + 64 (the pairs of the rotary embedding)
+__global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParams p, const float* __restrict__ part,
+                                                                 int qparts) {
   constexpr int Q = D / 8;                                                // threads per key row
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;           // over B * Hkv * Lk * D / 8
   const int64_t total = (int64_t)p.B * p.Hkv * p.Lk * Q;
@@ -702,10 +793,10 @@ __global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParam
   const int key = (idx / Q) % p.Lk;
   const int hk = (idx / ((int64_t)Q * p.Lk)) % p.Hkv;
   const int b = idx / ((int64_t)Q * p.Lk * p.Hkv);
-  const int64_t plane = (int64_t)p.B * p.Hq * p.Lk * D;
+  const int64_t plane = (int64_t)p.B * p.Hq * qparts * p.Lk * D;
   f32x4 sk1 = {0.f, 0.f, 0.f, 0.f}, sk2 = sk1, sv1 = sk1, sv2 = sk1;
-  for (int hg = 0; hg < p.group; hg++) {
-    const float* src = part + (((int64_t)b * p.Hq + hk * p.group + hg) * p.Lk + key) * D + 4 * d4;
+  for (int hg = 0; hg < p.group * qparts; hg++) {   // (query head of the group, part), in this fixed order
+    const float* src = part + ((((int64_t)b * p.Hkv + hk) * p.group * qparts + hg) * p.Lk + key) * D + 4 * d4;
     sk1 += *reinterpret_cast<const f32x4*>(src);
     sk2 += *reinterpret_cast<const f32x4*>(src + D / 2);
     sv1 += *reinterpret_cast<const f32x4*>(src + plane);
@@ -736,8 +827,36 @@ __global__ __launch_bounds__(256) void attn_bwd_group_sum_kernel(const AttnParam
 }
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
-inline size_t group_partials_bytes(int B, int Lk, int Hq, int Hkv) {
-  return Hq == Hkv ? 0 : align256((size_t)2 * B * Hq * Lk * D * sizeof(float));
+
+// Parts of the other side's range, for a kernel with `blocks` blocks that each walk `tiles` 64-row tiles.  As for the
+// forward's key split: with fewer blocks than it takes to keep the chip's 256 compute units busy and balanced -- one
+// block each when all are equally long, two each under a causal mask, where they are not and only a second, lighter
+// block per unit lets the heaviest-first order even that out -- the range is cut into 2 or 4 parts of at least 16
+// tiles (on average, when causal).
+inline int range_parts(int64_t blocks, int tiles, bool causal) {
+  const int64_t want = causal ? 512 : 256;
+  int s = 1;
+  while (s < 4 && blocks * s * 2 <= want && tiles >= 32 * s) s *= 2;
+  return s;
+}
+// dK/dV: parts of the query range of a (256-key block, query head)
+inline int query_parts(int B, int Lq, int Lk, int Hq, int Hkv, bool causal) {
+  const int64_t blocks = (int64_t)B * Hq * ((Lk + KV_BN - 1) / KV_BN);   // already one per QUERY head when they are split
+  return range_parts(blocks, (Lq + KV_BQ - 1) / KV_BQ, causal);
+}
+// dQ from kept dS: parts of the key range of a (256-query block, head)
+inline int key_parts(int B, int Lq, int Lk, int Hq, bool causal) {
+  return range_parts((int64_t)B * Hq * ((Lq + DQ_BM - 1) / DQ_BM), (Lk + 63) / 64, causal);
+}
+// fp32 partial dK / dV (grouped-query attention, or a split query range) and partial dQ (a split key range) share one
+// region: the first is summed up before the second is written.  Sized for the larger of the causal and the unmasked
+// policy, since the size query does not know the mask.
+inline size_t partials_bytes(int B, int Lq, int Lk, int Hq, int Hkv) {
+  const int qp = std::max(query_parts(B, Lq, Lk, Hq, Hkv, false), query_parts(B, Lq, Lk, Hq, Hkv, true));
+  const int kp = std::max(key_parts(B, Lq, Lk, Hq, false), key_parts(B, Lq, Lk, Hq, true));
+  const size_t kv = (Hq == Hkv && qp == 1) ? 0 : (size_t)2 * B * Hq * qp * Lk * D * sizeof(float);
+  const size_t dq = kp == 1 ? 0 : (size_t)kp * B * Lq * Hq * D * sizeof(float);
+  return align256(std::max(kv, dq));
 }
 
 }  // namespace
@@ -747,7 +866,7 @@ inline size_t group_partials_bytes(int B, int Lk, int Hq, int Hkv) {
 size_t ody_attn_bwd_pipe_workspace(int B, int Lq, int Lk, int Hq, int Hkv) {
   return align256(ody_attn_images_bytes(B, Lk, Hkv)) + 2 * align256(ody_attn_images_bytes(B, Lq, Hq)) +
          align256((size_t)B * Hq * ((Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)) +
-         group_partials_bytes(B, Lk, Hq, Hkv);
+         partials_bytes(B, Lq, Lk, Hq, Hkv);
 }
 
 size_t ody_attn_bwd_pipe_ds_bytes(int B, int Lq, int Lk, int Hq, int causal) {
@@ -779,28 +898,29 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
   if (!p.reuse_query_side && (rc = ody_launch_attn_bwd_prepass(p, qimg, doimg, stats, st))) return rc;
   if ((rc = ody_launch_attn_images(p.k, p.sk, p.B, p.Lk, p.Hkv, kimg, nullptr, 0, st))) return rc;
   const int key_blocks = (p.Lk + KV_BN - 1) / KV_BN;
-  if (p.group == 1) {
+  float* part = reinterpret_cast<float*>(
+      reinterpret_cast<unsigned char*>(stats) +
+      align256((size_t)p.B * p.Hq * ((p.Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)));
+  const int qparts = query_parts(p.B, p.Lq, p.Lk, p.Hq, p.Hkv, p.causal != 0);
+  if (p.group == 1 && qparts == 1) {
     if (p.ds)
       ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<false, true>), dim3(key_blocks * p.Hkv * p.B),
-                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr, 1);
     else
       ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<false, false>), dim3(key_blocks * p.Hkv * p.B),
-                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr);
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, nullptr, 1);
     if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
   } else {
-    float* part = reinterpret_cast<float*>(
-        reinterpret_cast<unsigned char*>(stats) +
-        align256((size_t)p.B * p.Hq * ((p.Lq + KV_BQ - 1) / KV_BQ) * KV_STAT_ELEMS * sizeof(bf16)));
     if (p.ds)
-      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, true>), dim3(key_blocks * p.Hq * p.B),
-                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, true>), dim3(key_blocks * p.Hq * qparts * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part, qparts);
     else
-      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, false>), dim3(key_blocks * p.Hq * p.B),
-                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part);
+      ODY_LAUNCH("attn_bwd_dkdv_pipe", st, (attn_bwd_dkdv_pipe_kernel<true, false>), dim3(key_blocks * p.Hq * qparts * p.B),
+                 dim3(KV_THREADS), smem_kv, p, qimg, doimg, stats, part, qparts);
     if ((rc = ody_check_launch("attn_bwd_dkdv_pipe"))) return rc;
     const int64_t n8 = (int64_t)p.B * p.Hkv * p.Lk * (D / 8);
     ODY_LAUNCH("attn_bwd_group_sum", st, attn_bwd_group_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p,
-               part);
+               part, qparts);
     if ((rc = ody_check_launch("attn_bwd_group_sum"))) return rc;
   }
   dim3 gq(((p.Lq + DQ_BM - 1) / DQ_BM) * p.Hq * p.B);
@@ -808,8 +928,13 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
     // what ody_attn_bwd_pipe_ds_bytes promised: whole 256-row blocks on both sides, queries and keys aligned
     ODY_REQUIRE(p.Lq % KV_BN == 0 && p.Lk % KV_BN == 0 && (!p.causal || p.off == 0) && KV_BN == DQ_BM, ODY_ERR_UNSUPPORTED,
                 "attn_bwd: kept dS needs multiples of %d rows on both sides and, if causal, as many keys as queries", KV_BN);
-    ODY_LAUNCH("attn_bwd_dq_kept", st, attn_bwd_dq_kept_kernel, gq, dim3(DQ_THREADS), smem_qs, p, kimg);
-    return ody_check_launch("attn_bwd_dq_kept");
+    const int kparts = key_parts(p.B, p.Lq, p.Lk, p.Hq, p.causal != 0);
+    ODY_LAUNCH("attn_bwd_dq_kept", st, attn_bwd_dq_kept_kernel, dim3(gq.x * kparts), dim3(DQ_THREADS), smem_qs, p, kimg, kparts,
+               part);
+    if ((rc = ody_check_launch("attn_bwd_dq_kept")) || kparts == 1) return rc;
+    const int64_t n8 = (int64_t)p.B * p.Lq * p.Hq * (D / 8);
+    ODY_LAUNCH("attn_bwd_dq_sum", st, attn_bwd_dq_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p, part, kparts);
+    return ody_check_launch("attn_bwd_dq_sum");
   }
   ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
   return ody_check_launch("attn_bwd_dq_pipe");

@@ -320,6 +320,57 @@ def test_attention_bwd_kept_ds_full_blocks(case, dev):
     assert_parity(dq2, dq_ref, TOL_BF16, "dq of the recomputing kernel", 1e-3)
 
 
+@pytest.mark.parametrize("case", [(1, 4096, 512, 2, 2, False, True, False), (1, 512, 4096, 2, 2, False, False, True),
+                                  (1, 4096, 4096, 2, 1, True, True, True), (1, 4096, 4096, 2, 2, True, True, True),
+                                  (1, 4100, 600, 2, 2, False, True, False), (2, 2304, 2304, 1, 1, True, True, True)],
+                         ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d_kv%d_q%d" % c)
+def test_attention_bwd_range_parts(case, dev):
+    """Few key blocks against many queries, or few query blocks against many keys (the steps of a ring over short
+    blocks): the dK/dV kernel cuts each block's query range, the dQ kernel over kept dS each block's key range, into
+    parts that leave fp32 partial sums, and a second kernel adds them up.  Every destination of dq, against the oracle."""
+    from odysseus_transformer_amd import ops, _lib
+    B, Lq, Lk, Hq, Hkv, causal, kv_parts, q_parts = case
+    print(f"range parts case={case}", flush=True)
+    keep = Lq % 256 == 0 and Lk % 256 == 0
+    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, 128, torch.bfloat16, seed=Lq + 3 * Lk)
+    o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal)
+    dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float(), causal=causal)
+    qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
+    o, lse = ops.attn_fwd(qg, kg, vg, causal=causal)
+    _lib.profile_enable(True)
+    try:
+        dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=keep)
+        torch.cuda.synchronize()
+        ran = set(_lib.profile_collect())
+    finally:
+        _lib.profile_enable(False)
+    assert ("attn_bwd_group_sum" in ran) == kv_parts and ("attn_bwd_dq_sum" in ran) == q_parts, ran
+    assert_parity(dq, dq_ref, TOL_BF16, "dq", 1e-3)
+    assert_parity(dk, dk_ref, TOL_BF16, "dk", 1e-3)
+    assert_parity(dv, dv_ref, TOL_BF16, "dv")
+    # the partial sums do not depend on the order in which the blocks ran
+    dq_b, dk_b, dv_b = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=keep)
+    assert torch.equal(dq_b, dq) and torch.equal(dk_b, dk) and torch.equal(dv_b, dv)
+    if keep:   # the same dK / dV from the recomputing dQ kernel's side of the library
+        _, dk_r, dv_r = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=False)
+        assert torch.equal(dk_r, dk) and torch.equal(dv_r, dv)
+    acc0 = randn((B, Lq, Hq, 128), 5).to(dev)
+    acc = acc0.clone()
+    ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=acc, accumulate_dq=True, keep_ds=keep)
+    assert_parity((acc - acc0).cpu(), dq_ref, TOL_BF16, "dq added to an fp32 buffer", 1e-3)
+    accb = acc0.to(torch.bfloat16)
+    ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=accb, accumulate_dq=True, keep_ds=keep)
+    assert_parity(accb, acc0.to(torch.bfloat16).float().cpu() + dq_ref, TOL_BF16, "dq added to a bf16 buffer")
+    pos_q = (torch.arange(Lq, device=dev) + (Lk - Lq if causal else 0)).repeat(B, 1)
+    pos_k = torch.arange(Lk, device=dev).repeat(B, 1)
+    tq, tk = ops.rope_table(pos_q, B * Lq, 128, 10000.0), ops.rope_table(pos_k, B * Lk, 128, 10000.0)
+    dq_r, dk_r, _ = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, rope_tables=(tq, tk), keep_ds=keep)
+    cq, sq = oracle.rope_cos_sin(pos_q.cpu(), 128, 10000.0)
+    ck, sk = oracle.rope_cos_sin(pos_k.cpu(), 128, 10000.0)
+    assert_parity(dq_r, oracle.apply_rope_bwd(dq_ref, cq, sq), TOL_BF16, "dq rotated back", 1e-3)
+    assert_parity(dk_r, oracle.apply_rope_bwd(dk_ref, ck, sk), TOL_BF16, "dk rotated back", 1e-3)
+
+
 @pytest.mark.parametrize("case", [(1, 512, 4096, 2, 2, 4, False), (1, 300, 2100, 4, 1, 4, False), (2, 256, 1100, 2, 2, 2, False),
                                   (1, 2048, 1024, 4, 4, 2, False), (1, 2048, 2048, 4, 4, 4, True), (1, 1100, 1500, 2, 1, 2, True)],
                          ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_parts%d_c%d" % c)
