@@ -607,9 +607,18 @@ def layer_share(_lib, ops, rn, dev, attn_sec):
         prof = _lib.profile_collect()
         _lib.profile_enable(False)
         tk = sum(total_ms for (_, total_ms, _) in prof.values()) / 10 * 1e-3
+        # same-box yardstick: a device copy that moves the same number of bytes (half read, half written), one
+        # launch between two HIP events like the kernels above (measurement only, on no product path)
+        src = torch.empty(nbytes // 2, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        ty = spread(time_events(lambda: dst.copy_(src), 20, 3))["median"] * 1e-3
+        del src, dst
         res[tag] = {"ms": round(t * 1e3, 4), "kernel_ms": round(tk * 1e3, 4), "kernels": sorted(prof),
                     "algorithmic_GBs": round(nbytes / tk / 1e9, 1),
-                    "frac_of_hbm_peak": round(nbytes / tk / 1e9 / PEAK_HBM_GBS, 3)}
+                    "frac_of_hbm_peak": round(nbytes / tk / 1e9 / PEAK_HBM_GBS, 3),
+                    "copy_yardstick": {"ms": round(ty * 1e3, 4), "GBs": round(nbytes / ty / 1e9, 1),
+                                       "frac_of_hbm_peak": round(nbytes / ty / 1e9 / PEAK_HBM_GBS, 3),
+                                       "ours_over_yardstick": round(ty / tk, 3)}}
         return t
 
     t_attn_half = attn_sec
@@ -659,7 +668,7 @@ def layer_share(_lib, ops, rn, dev, attn_sec):
     membound("rope", lambda: ops.rope_(qkv, H + HKV), 2 * 4 * L * (H + HKV) * D * e)
     del qkv
     for k in ("rmsnorm_fwd", "rmsnorm_bwd", "rope"):
-        big[k] = {n: res[k][n] for n in ("kernel_ms", "algorithmic_GBs", "frac_of_hbm_peak")}
+        big[k] = {n: res[k][n] for n in ("kernel_ms", "algorithmic_GBs", "frac_of_hbm_peak", "copy_yardstick")}
     res.clear()
     res.update(keep)
     res["memory_bound_at_8x_rows"] = {"rows": {"rmsnorm": T8, "rope": 4 * L}, **big}

@@ -8,6 +8,16 @@ namespace {
 
 using namespace tile128;
 
+// an image leaves by a streaming store: this kernel does not read it again
+__device__ __forceinline__ void store_image_chunk(bf16* p, bf16x8 v) {
+  typedef unsigned raw_t __attribute__((ext_vector_type(4)));
+#ifdef ODY_PLAIN_STORES
+  *reinterpret_cast<bf16x8*>(p) = v;
+#else
+  __builtin_nontemporal_store(__builtin_bit_cast(raw_t, v), reinterpret_cast<raw_t*>(p));
+#endif
+}
+
 __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict__ src, AttnStrides s, int L,
                                                           bf16* __restrict__ dst, int ntiles, int H,
                                                           int* __restrict__ flags, int nflags) {
@@ -38,7 +48,7 @@ __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict
       const int row = 32 * (e >> 2) + 16 * g + 4 * (e & 3) + ss + 2 * kt;
       v[e] = tile[row * PITCH + d];
     }
-    *reinterpret_cast<bf16x8*>(img + q * 8) = v;
+    store_image_chunk(img + q * 8, v);
   }
 }
 
@@ -96,7 +106,7 @@ __global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams 
         const int row = 32 * (e >> 2) + 16 * g + 4 * (e & 3) + ss + 2 * kt;
         v[e] = tile[row * PITCH + d];
       }
-      *reinterpret_cast<bf16x8*>(img + q * 8) = v;
+      store_image_chunk(img + q * 8, v);
     }
   }
   if (tid < 128) {
