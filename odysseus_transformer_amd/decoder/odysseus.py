@@ -140,10 +140,12 @@ class LlamaFlashAttention2TPSP(nn.Module):
                 "`static` cache implementation is not compatible with `attn_implementation==flash_attention_2` "
                 "make sure to use `sdpa` in the mean time, and open an issue at "
                 "https://github.com/huggingface/transformers")
-        if attention_mask is not None:
-            raise NotImplementedError("padding masks are not supported: the training loop passes attention_mask=None")
         bsz, local_q_len, _ = hidden_states.size()
         assert bsz == 1, f"bsz: {bsz}"
+        # the training path: no padding and nothing in the cache yet.  A padding mask or earlier cache content takes
+        # the general path below, as decoder/odysseus.py:215-263 hands both on to the host's flash-attention call.
+        cached = past_key_value is not None and past_key_value.get_seq_length(self.layer_idx) > 0
+        general = cached or attention_mask is not None
         if self.training and self.attention_dropout != 0.0:
             raise NotImplementedError("attention dropout is not implemented (the reference trains with 0.0)")
         scale = 1.0 / math.sqrt(self.head_dim)
@@ -153,7 +155,12 @@ class LlamaFlashAttention2TPSP(nn.Module):
             q_len = local_q_len * get_model_parallel_world_size()
             if not self.sequence_parallel:
                 hidden_states = allgather_bsz1(hidden_states)
-            if self._can_fuse_rope(hidden_states):
+            if general:
+                qkv = self.qkv_proj(hidden_states).view(bsz, q_len, nh + 2 * nkv, D)
+                qkv = ops.apply_rope_packed(qkv, nh + nkv, position_ids, self.rope_theta)
+                attn_output = self._attend_general(qkv[:, :, :nh], qkv[:, :, nh:nh + nkv], qkv[:, :, nh + nkv:],
+                                                   attention_mask, past_key_value, cache_position, scale)
+            elif self._can_fuse_rope(hidden_states):
                 # projection, rotary embedding and attention as one autograd node: the rotation rides in the
                 # projection's epilogue, its backward in the epilogues of the attention backward
                 qkv3, attn_output, _ = ops.QKVRoPEAttnFunc.apply(hidden_states, self.qkv_proj.weight, nh, nkv, D,
@@ -161,7 +168,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
             else:
                 qkv3, attn_output, _ = PackedRoPEAttnFunc.apply(self.qkv_proj(hidden_states), nh, nkv, D, position_ids,
                                                                 self.rope_theta, scale)
-            if past_key_value is not None:
+            if past_key_value is not None and not general:
                 qkv = qkv3.detach().view(bsz, q_len, nh + 2 * nkv, D)
                 self._update_cache(past_key_value, qkv[:, :, nh:nh + nkv], qkv[:, :, nh + nkv:], q_len, cache_position)
         else:
@@ -172,9 +179,12 @@ class LlamaFlashAttention2TPSP(nn.Module):
             v = self.v_proj(hidden_states).view(bsz, q_len, nkv, D)
             q = ops.apply_rope_packed(q, nh, position_ids, self.rope_theta)
             k = ops.apply_rope_packed(k, nkv, position_ids, self.rope_theta)
-            if past_key_value is not None:
-                self._update_cache(past_key_value, k.detach(), v.detach(), q_len, cache_position)
-            attn_output = ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+            if general:
+                attn_output = self._attend_general(q, k, v, attention_mask, past_key_value, cache_position, scale)
+            else:
+                if past_key_value is not None:
+                    self._update_cache(past_key_value, k.detach(), v.detach(), q_len, cache_position)
+                attn_output = ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
 
         attn_output = attn_output.reshape(bsz, q_len, nh * D)
         residual = kwargs.get("residual")
@@ -209,13 +219,39 @@ class LlamaFlashAttention2TPSP(nn.Module):
                 and not torch.is_autocast_enabled("cuda"))
 
     def _update_cache(self, cache, k, v, q_len, cache_position):
-        """Hands the rotated keys and the values of a prefill to the caller's cache, as
-        decoder/odysseus.py:215-220 does.  Attending to EARLIER cache content is the
-        decoding path, which this training-side module does not implement."""
+        """Hands the rotated keys and the values of a prefill into an EMPTY cache to the caller's cache, as
+        decoder/odysseus.py:215-220 does; the attention itself then needs nothing back from it."""
         k_all, _ = cache.update(k.transpose(1, 2), v.transpose(1, 2), self.layer_idx,
                                 {"cache_position": cache_position})
-        if k_all.shape[-2] != q_len:
-            raise NotImplementedError("attention over a non-empty KV cache (incremental decoding) is not implemented")
+        assert k_all.shape[-2] == q_len, "the cache was not empty"
+
+    def _attend_general(self, q, k, v, attention_mask, cache, cache_position, scale):
+        """Attention of the rotated q (1, Lq, nh, D) over k, v (1, Lq, nkv, D) appended to the cache's earlier
+        content, with an optional padding mask (1, Lk) of 0 / 1 over all keys -- what decoder/odysseus.py:215-263
+        reaches through the cache's update() and the host's flash-attention forward: queries sit at the END of
+        the keys (query i sees keys up to i + Lk - Lq), masked-out tokens take no part on either side and their
+        output rows are zero (the unpad / varlen / pad sequence of the host collapses to one gather and one
+        scatter at batch size 1)."""
+        if cache is not None:
+            k_all, v_all = cache.update(k.transpose(1, 2), v.transpose(1, 2), self.layer_idx,
+                                        {"cache_position": cache_position})
+            k, v = k_all.transpose(1, 2), v_all.transpose(1, 2)
+        Lq, Lk = q.shape[1], k.shape[1]
+        if attention_mask is None:
+            return ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+        if attention_mask.dim() != 2 or attention_mask.shape[0] != 1 or attention_mask.shape[1] != Lk:
+            raise ValueError(f"attention_mask must be a (1, {Lk}) padding mask over the keys; got {tuple(attention_mask.shape)}")
+        keep_k = attention_mask[0] != 0
+        idx_k = keep_k.nonzero().squeeze(1)
+        # queries are the last Lq key positions; a single decoding query is always kept (as the host's unpad does)
+        idx_q = idx_k.new_zeros(1) if Lq == 1 else keep_k[Lk - Lq:].nonzero().squeeze(1)
+        if idx_k.numel() == Lk and idx_q.numel() == Lq:
+            return ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+        if idx_q.numel() == 0 or idx_k.numel() == 0:
+            return q * 0
+        o = ops.flash_attn_func(q.index_select(1, idx_q), k.index_select(1, idx_k), v.index_select(1, idx_k), 0.0,
+                                softmax_scale=scale, causal=True)
+        return torch.zeros_like(q).index_copy(1, idx_q, o)
 
 
 class LlamaMLPZeRO(nn.Module):

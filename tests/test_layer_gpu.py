@@ -320,3 +320,87 @@ def test_zigzag_ring_patch_on_a_mistral_host(dev):
         logits = model(ids.to(dev), position_ids=pos.to(dev), use_cache=False).logits
     # bf16 weights and activations against the fp32 host: the bar of a whole bf16 model, not of one kernel
     assert rel_err(logits, ref) <= 5e-2
+
+
+@pytest.mark.parametrize("pack_weight", [True, False], ids=["packed", "unpacked"])
+def test_attention_block_with_a_padding_mask(pack_weight, dev):
+    """A (1, L) padding mask (decoder/odysseus.py:256-263 hands it to the host's flash-attention forward, which
+    drops the masked tokens, attends over the rest and pads the result with zeros): the kept tokens get what the
+    oracle computes on the kept tokens alone, at their own positions; masked tokens get zero rows and send no
+    gradient anywhere."""
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    d, H, Hkv, D, L = 512, 4, 2, 128, 300
+    dt = torch.bfloat16
+    attn = LlamaFlashAttention2TPSP(_config(d, H, Hkv, D, 1024), 0, pack_weight=pack_weight).to(dt).to(dev)
+    w = randn(((H + 2 * Hkv) * D, d), 17, std=0.02, dtype=dt)
+    wo = randn((d, H * D), 18, std=0.02, dtype=dt)
+    with torch.no_grad():
+        if pack_weight:
+            attn.qkv_proj.weight.copy_(w)
+        else:
+            attn.q_proj.weight.copy_(w[:H * D])
+            attn.k_proj.weight.copy_(w[H * D:(H + Hkv) * D])
+            attn.v_proj.weight.copy_(w[(H + Hkv) * D:])
+        attn.o_proj.weight.copy_(wo)
+    x = randn((1, L, d), 19, dtype=dt)
+    mask = torch.ones(1, L, dtype=torch.long)
+    mask[0, :37] = 0          # left padding
+    mask[0, 150:161] = 0      # and a hole
+    keep = mask[0].nonzero().squeeze(1)
+    pos = (mask.cumsum(1) - 1).clamp(min=0)       # the positions a host derives from the mask
+    xg = x.to(dev).requires_grad_(True)
+    y = attn(xg, attention_mask=mask.to(dev), position_ids=pos.to(dev))[0]
+    dy = randn((1, L, d), 20, dtype=dt)
+    y.backward(dy.to(dev))
+    xr = x.float()[:, keep].requires_grad_(True)
+    y_ref, _ = oracle.attention_block(xr, w.float(), wo.float(), H, Hkv, D, position_ids=pos[:, keep], differentiable=True)
+    y_ref.backward(dy.float()[:, keep])
+    assert_parity(y[:, keep.to(dev)], y_ref.detach(), TOL_BF16, "kept rows")
+    gone = (mask[0] == 0).nonzero().squeeze(1).to(dev)
+    assert torch.count_nonzero(y[:, gone]) == 0 and torch.count_nonzero(xg.grad[:, gone]) == 0
+    assert_parity(xg.grad[:, keep.to(dev)], xr.grad, TOL_BF16, "dx of the kept rows", 1e-3)
+    # a mask without zeros is the unmasked call
+    y_all = attn(xg.detach(), attention_mask=torch.ones(1, L, dtype=torch.long, device=dev))[0]
+    assert torch.equal(y_all, attn(xg.detach())[0])
+    with pytest.raises(ValueError):
+        attn(xg.detach(), attention_mask=torch.ones(1, L + 1, dtype=torch.long, device=dev))
+
+
+def test_attention_block_decodes_from_a_kv_cache(dev):
+    """Prefill into the host's DynamicCache, then more tokens against the cached keys (decoder/odysseus.py:215-220):
+    every step gives the rows that the oracle computes for the whole sequence at once."""
+    from transformers import DynamicCache
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    d, H, Hkv, D, L0 = 512, 4, 2, 128, 200
+    dt = torch.bfloat16
+    attn = LlamaFlashAttention2TPSP(_config(d, H, Hkv, D, 1024), 0).to(dt).to(dev).eval()
+    w = randn(((H + 2 * Hkv) * D, d), 27, std=0.02, dtype=dt)
+    wo = randn((d, H * D), 28, std=0.02, dtype=dt)
+    with torch.no_grad():
+        attn.qkv_proj.weight.copy_(w)
+        attn.o_proj.weight.copy_(wo)
+    steps = [L0, 1, 1, 7, 1]                      # prefill, single tokens, a chunk of 7
+    L = sum(steps)
+    x = randn((1, L, d), 29, dtype=dt)
+    y_ref, _ = oracle.attention_block(x.float(), w.float(), wo.float(), H, Hkv, D)
+    cache = DynamicCache()
+    at = 0
+    with torch.no_grad():
+        for n in steps:
+            pos = torch.arange(at, at + n, device=dev)[None]
+            y, _, c = attn(x[:, at:at + n].to(dev), position_ids=pos, past_key_value=cache, use_cache=True, cache_position=pos[0])
+            assert c is cache and cache.get_seq_length(0) == at + n
+            assert_parity(y, y_ref[:, at:at + n], TOL_BF16, f"rows {at}..{at + n}", 1e-3)
+            at += n
+    # with a padding mask over cached and new keys: the masked cache entries take no part
+    mask = torch.ones(1, L + 1, dtype=torch.long)
+    mask[0, :5] = 0
+    xn = randn((1, 1, d), 30, dtype=dt)
+    pos = torch.tensor([[L - 5]], device=dev)
+    with torch.no_grad():
+        y = attn(xn.to(dev), attention_mask=mask.to(dev), position_ids=pos, past_key_value=cache, use_cache=True)[0]
+    # oracle: the kept tokens 5..L-1 at positions 5..L-1 as they were cached, the new one at position L - 5
+    xs = torch.cat([x.float()[:, 5:], xn.float()], 1)
+    ps = torch.cat([torch.arange(5, L), torch.tensor([L - 5])])[None]
+    y2, _ = oracle.attention_block(xs, w.float(), wo.float(), H, Hkv, D, position_ids=ps)
+    assert_parity(y, y2[:, -1:], TOL_BF16, "masked decode step", 1e-3)
