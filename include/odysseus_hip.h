@@ -76,7 +76,11 @@ int ody_profile_collect(char* out, size_t cap);
  * pointer, strides that are multiples of 16 bytes (8 bf16 / 4 fp32 elements).
  * workspace: ody_attn_fwd_workspace_bytes(...) bytes, 256-byte aligned (the bf16
  * head_dim-128 kernel keeps a transposed copy of V and one int per 256-query block
- * there; 0 bytes = may be NULL).
+ * there; 0 bytes = may be NULL).  For a call with too few 256-query blocks to fill the
+ * chip (a ring step of few queries against a long key block) the size includes fp32
+ * partial results: the kernel then cuts every block's key range into 2 or 4 parts and a
+ * second kernel merges them by their log-sum-exp.  A workspace with room for the V copy
+ * and the flags only is accepted too; such a call runs unsplit.
  */
 size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
@@ -90,12 +94,15 @@ int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* 
 
 /* ody_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
- * attention routine allocates through PyTorch.  Same arguments and results as ody_attn_fwd, bit
- * for bit, without the workspace: the scratch of the bf16 head_dim-128 kernel (transposed image of
- * V, block flags) lives in a buffer of ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES that the library itself
- * holds on every GPU it runs on, for the life of the process.  The call allocates and frees
- * nothing and synchronises nothing; a shape whose ody_attn_fwd_workspace_bytes exceeds the buffer
- * (more than about 131000 key rows over all kv heads and batches) returns ODY_ERR_WORKSPACE.
+ * attention routine allocates through PyTorch.  Same arguments and results as ody_attn_fwd, without
+ * the workspace: the scratch of the bf16 head_dim-128 kernel (transposed image of V, block flags,
+ * the fp32 parts of a call that cuts its key range) lives in a buffer of
+ * ODY_ATTN_FWD_NOALLOC_SCRATCH_BYTES that the library itself holds on every GPU it runs on, for
+ * the life of the process.  Bit for bit the results of ody_attn_fwd with a workspace of the same
+ * kind: a call whose fp32 parts do not fit the buffer runs unsplit (as ody_attn_fwd does with a
+ * workspace without room for them).  The call allocates and frees nothing and synchronises
+ * nothing; a shape whose V image and flags exceed the buffer (more than about 131000 key rows
+ * over all kv heads and batches) returns ODY_ERR_WORKSPACE.
  * All calls on one GPU share that GPU's buffer: calls that may overlap there (different
  * streams, different threads) race, so keep them on one stream or order them with events.  The
  * first call on a device looks up the buffer's address; make that call outside graph capture.
@@ -132,7 +139,9 @@ int ody_attn_fwd_noalloc(const void* q, const void* k, const void* v, void* out,
  *                             2 bytes per visible (query, key) pair: about B * Hq * Lq * Lk bytes when causal,
  *                             twice that for a full block.
  * workspace: ody_attn_bwd_workspace_bytes(...) bytes, 256-byte aligned (delta, and for
- * the bf16 head_dim-128 kernels transposed copies of K, Q and dO).
+ * the bf16 head_dim-128 kernels transposed copies of K, Q and dO, plus fp32 partial dK / dV
+ * or dQ where grouped-query attention, or a call with one short side, is cut into parts
+ * that a second kernel adds up in a fixed order).
  */
 enum ody_attn_bwd_flags { ODY_BWD_ACCUMULATE_DQ = 1, ODY_BWD_DQ_F32 = 2, ODY_BWD_REUSE_QUERY_SIDE = 4, ODY_BWD_KEEP_DS = 8 };
 size_t ody_attn_bwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
