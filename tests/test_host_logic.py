@@ -100,7 +100,7 @@ def test_attention_module_surface():
         m(torch.zeros(2, 4, 64))
     with pytest.raises(RuntimeError, match="HIP device"):     # CPU tensors are refused: no fallback path
         m(torch.zeros(1, 4, 64))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="HIP device"):     # a padding mask takes the general path, which needs the GPU too
         m(torch.zeros(1, 4, 64), attention_mask=torch.ones(1, 4))
 
 
