@@ -82,14 +82,34 @@ __device__ __forceinline__ void store_dq_row(const AttnParams& p, const f32x16 (
   }
 }
 
+// The same accumulators as one part's unscaled fp32 sum (a dQ kernel whose key range is cut into parts):
+// dq_part [part][B][Lq][Hq][D]; attn_bwd_dq_sum_kernel adds the parts and finishes dq as store_dq_row would.
+__device__ __forceinline__ void store_dq_part(float* __restrict__ dq_part, int part, const AttnParams& p,
+                                              const f32x16 (&dq)[DT], int b, int h, int qi, int g) {
+  if (qi >= p.Lq) return;
+  float* dst = dq_part + ((((int64_t)part * p.B + b) * p.Lq + qi) * p.Hq + h) * D;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+      f32x4 w;
+#pragma unroll
+      for (int e = 0; e < 4; e++) w[e] = dq[dt][4 * a + e];
+      *reinterpret_cast<f32x4*>(dst + 32 * dt + 8 * a + 4 * g) = w;
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------
 constexpr int DQ_QT = 1, DQ_WAVES = 8, DQ_BM = 32 * DQ_QT * DQ_WAVES, DQ_THREADS = 64 * DQ_WAVES;
 static_assert(DQ_WAVES == 8, "the load split and the vmcnt waits assume 8 wavefronts");
 
+// kparts > 1 (too few query blocks for the chip): block id = part + kparts * (the usual id), the block takes part
+// `part` of its key tiles and leaves its unscaled fp32 sum in dq_part.
 __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const AttnParams p,
-                                                                       const bf16* __restrict__ kimg) {
+                                                                       const bf16* __restrict__ kimg, int kparts,
+                                                                       float* __restrict__ dq_part) {
   constexpr int BN = 64, QT = DQ_QT;
   constexpr int STAGE = 2 * TILE_ELEMS + IMG_ELEMS;   // K tile, V tile, K^T image
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -98,8 +118,9 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g = lane >> 5,
             i = lane & 31;
   simd_stagger(tid);
-  const BlockCoord bc = ody_block_coord(p.Hq, p.B);
-  const int nqb = gridDim.x / (p.Hq * p.B);
+  const int kpart = blockIdx.x % kparts;
+  const BlockCoord bc = ody_block_coord_of(blockIdx.x / kparts, p.Hq, p.B);
+  const int nqb = gridDim.x / (p.Hq * p.B * kparts);
   const int qblk = p.causal ? (nqb - 1 - bc.rank) : bc.rank;   // heaviest blocks first
   const int h = bc.h, b = bc.b, hk = h / p.group;
   const int q0 = qblk * DQ_BM, wq0 = q0 + wave * 32 * QT;
@@ -114,10 +135,16 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
   const int q_hi = min(q0 + DQ_BM, p.Lq) - 1;
   int n_end = p.causal ? min(p.Lk, q_hi + p.off + 1) : p.Lk;
   if (n_end < 0) n_end = 0;
-  const int ntiles = (n_end + BN - 1) / BN;
+  int ntiles = (n_end + BN - 1) / BN;
   int n_full = p.Lk / BN;   // tiles [0, n_full) need no mask for any wavefront of the block
   if (p.causal) n_full = min(n_full, max(0, (q0 + p.off + 1) / BN));
   n_full = min(n_full, ntiles);
+  int t_first = 0;   // this block's part of the tiles: [t_first, ntiles)
+  if (kparts > 1) {
+    const int per = (ntiles + kparts - 1) / kparts;
+    t_first = min(kpart * per, ntiles);
+    ntiles = min(t_first + per, ntiles);
+  }
 
   auto load_part = [&](bf16* st, int t, int j) {   // j = 0, 1: the two halves of a stage's loads
     {
@@ -137,8 +164,8 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
     load_part(st, t, 0);
     load_part(st, t, 1);
   };
-  if (ntiles > 0) load_stage(ring, 0);
-  if (ntiles > 1) load_stage(ring + STAGE, 1);
+  if (t_first < ntiles) load_stage(ring, t_first);
+  if (t_first + 1 < ntiles) load_stage(ring + STAGE, t_first + 1);
 
   bf16x8 qf[QT][KS], dof[QT][KS];
   float lse2[QT], delta[QT];
@@ -244,21 +271,22 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_pipe_kernel(const Attn
     }
   };
 
-  for (int t = 0; t < ntiles; t++) {
+  for (int t = t_first; t < ntiles; t++) {
     // stage t landed (the loads of stage t+1 may still be in flight), everyone done with stage t-1
     if (t + 1 < ntiles) {
       asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
     } else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    const bf16* st = ring + (t % 3) * STAGE;
+    const bf16* st = ring + ((t - t_first) % 3) * STAGE;
     const bool dead = p.causal && t * BN > wq0 + 32 * QT - 1 + p.off;   // every key of the tile is after this wavefront's queries
     if (!dead) tile(st, t, t >= n_full);
     // the loads go last: issuing them costs this wavefront time, and here it would otherwise wait at the barrier
-    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 0);
-    if (t + 2 < ntiles) load_part(ring + ((t + 2) % 3) * STAGE, t + 2, 1);
+    if (t + 2 < ntiles) load_part(ring + ((t + 2 - t_first) % 3) * STAGE, t + 2, 0);
+    if (t + 2 < ntiles) load_part(ring + ((t + 2 - t_first) % 3) * STAGE, t + 2, 1);
   }
 
-  store_dq_row(p, dq[0], b, h, wq0 + i, g);
+  if (kparts > 1) store_dq_part(dq_part, kpart, p, dq[0], b, h, wq0 + i, g);
+  else store_dq_row(p, dq[0], b, h, wq0 + i, g);
 }
 
 // ---------------------------------------------------------------------------------
@@ -619,18 +647,7 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
   }
   // position 32 mt + i of the tile's kept order = chunk 4 mt + (i >> 3), element i & 7
   const int qrow = qblk * DQ_BM + KV_BQ * x + 32 * ((i >> 2) & 1) + 16 * ((i >> 3) & 1) + 4 * (i & 3) + (i >> 4) + 2 * mt;
-  auto store_part = [&](const f32x16 (&acc)[DT]) {
-    float* dst = dq_part + ((((int64_t)kpart * p.B + b) * p.Lq + qrow) * p.Hq + h) * D;
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-      for (int a = 0; a < 4; a++) {
-        f32x4 w;
-#pragma unroll
-        for (int e = 0; e < 4; e++) w[e] = acc[dt][4 * a + e];
-        *reinterpret_cast<f32x4*>(dst + 32 * dt + 8 * a + 4 * g) = w;
-      }
-  };
+  auto store_part = [&](const f32x16 (&acc)[DT]) { store_dq_part(dq_part, kpart, p, acc, b, h, qrow, g); };
 
   u32x4 regs[DQK_SETS][6];
   // tile t: this wavefront's 4 of the 32 pieces (x, c) of key tile t & 3 of block (t >> 2, qblk) -- 32 KB in a row --
@@ -727,7 +744,7 @@ __global__ __launch_bounds__(DQ_THREADS) void attn_bwd_dq_kept_kernel(const Attn
   else store_dq_row(p, dq, b, h, qrow, g);
 }
 
-// dq = the sum of the fp32 parts of a key-split attn_bwd_dq_kept_kernel, finished like store_dq_row does; one thread per
+// dq = the sum of the fp32 parts of a key-split dQ kernel, finished like store_dq_row does; one thread per
 // 4 elements d..d+3 of the first half of a (query, head) row and their partners d + 64 (the pairs of the rotary
 // embedding)
 __global__ __launch_bounds__(256) void attn_bwd_dq_sum_kernel(const AttnParams p, const float* __restrict__ dq_part, int kparts) {
@@ -844,7 +861,7 @@ inline int query_parts(int B, int Lq, int Lk, int Hq, int Hkv, bool causal) {
   const int64_t blocks = (int64_t)B * Hq * ((Lk + KV_BN - 1) / KV_BN);   // already one per QUERY head when they are split
   return range_parts(blocks, (Lq + KV_BQ - 1) / KV_BQ, causal);
 }
-// dQ from kept dS: parts of the key range of a (256-query block, head)
+// dQ (either kernel): parts of the key range of a (256-query block, head)
 inline int key_parts(int B, int Lq, int Lk, int Hq, bool causal) {
   return range_parts((int64_t)B * Hq * ((Lq + DQ_BM - 1) / DQ_BM), (Lk + 63) / 64, causal);
 }
@@ -936,6 +953,11 @@ int ody_launch_attn_bwd_pipe(const AttnParams& p, void* workspace, hipStream_t s
     ODY_LAUNCH("attn_bwd_dq_sum", st, attn_bwd_dq_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p, part, kparts);
     return ody_check_launch("attn_bwd_dq_sum");
   }
-  ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, gq, dim3(DQ_THREADS), smem_q, p, kimg);
-  return ody_check_launch("attn_bwd_dq_pipe");
+  const int kparts = key_parts(p.B, p.Lq, p.Lk, p.Hq, p.causal != 0);
+  ODY_LAUNCH("attn_bwd_dq_pipe", st, attn_bwd_dq_pipe_kernel, dim3(gq.x * kparts), dim3(DQ_THREADS), smem_q, p, kimg, kparts,
+             part);
+  if ((rc = ody_check_launch("attn_bwd_dq_pipe")) || kparts == 1) return rc;
+  const int64_t n8 = (int64_t)p.B * p.Lq * p.Hq * (D / 8);
+  ODY_LAUNCH("attn_bwd_dq_sum", st, attn_bwd_dq_sum_kernel, dim3((unsigned)((n8 + 255) / 256)), dim3(256), 0, p, part, kparts);
+  return ody_check_launch("attn_bwd_dq_sum");
 }

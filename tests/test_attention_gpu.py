@@ -322,7 +322,8 @@ def test_attention_bwd_kept_ds_full_blocks(case, dev):
 
 @pytest.mark.parametrize("case", [(1, 4096, 512, 2, 2, False, True, False), (1, 512, 4096, 2, 2, False, False, True),
                                   (1, 4096, 4096, 2, 1, True, True, True), (1, 4096, 4096, 2, 2, True, True, True),
-                                  (1, 4100, 600, 2, 2, False, True, False), (2, 2304, 2304, 1, 1, True, True, True)],
+                                  (1, 4100, 600, 2, 2, False, True, False), (2, 2304, 2304, 1, 1, True, True, True),
+                                  (1, 500, 4200, 2, 1, False, True, True), (1, 4100, 4100, 2, 2, True, True, True)],
                          ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d_kv%d_q%d" % c)
 def test_attention_bwd_range_parts(case, dev):
     """Few key blocks against many queries, or few query blocks against many keys (the steps of a ring over short
@@ -351,9 +352,17 @@ def test_attention_bwd_range_parts(case, dev):
     # the partial sums do not depend on the order in which the blocks ran
     dq_b, dk_b, dv_b = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=keep)
     assert torch.equal(dq_b, dq) and torch.equal(dk_b, dk) and torch.equal(dv_b, dv)
-    if keep:   # the same dK / dV from the recomputing dQ kernel's side of the library
-        _, dk_r, dv_r = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=False)
+    if keep:   # the recomputing dQ kernel cuts its key range the same way; dK / dV do not depend on which dQ kernel runs
+        _lib.profile_enable(True)
+        try:
+            dq_r, dk_r, dv_r = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, keep_ds=False)
+            torch.cuda.synchronize()
+            ran = set(_lib.profile_collect())
+        finally:
+            _lib.profile_enable(False)
+        assert "attn_bwd_dq_pipe" in ran and ("attn_bwd_dq_sum" in ran) == q_parts, ran
         assert torch.equal(dk_r, dk) and torch.equal(dv_r, dv)
+        assert_parity(dq_r, dq_ref, TOL_BF16, "dq of the recomputing kernel", 1e-3)
     acc0 = randn((B, Lq, Hq, 128), 5).to(dev)
     acc = acc0.clone()
     ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=acc, accumulate_dq=True, keep_ds=keep)
