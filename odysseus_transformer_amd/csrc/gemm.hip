@@ -64,6 +64,17 @@ struct OperandTile {
       return concat4(lds_read_tr16(p), lds_read_tr16(p + 4 * PITCH));
     }
   }
+  // The same for the 16 x 16 x 32 MFMA: tile rows [r16, r16 + 16), k-step ks (32 K values): lane l gets row
+  // r16 + (l & 15), k = 32 ks + 8 (l >> 4) .. + 7
+  __device__ static __forceinline__ bf16x8 frag16(const bf16* lds, int r16, int ks, int lane) {
+    const int c = lane & 15, q = lane >> 4;
+    if (KC) {
+      return *reinterpret_cast<const bf16x8*>(lds + (r16 + c) * PITCH + 32 * ks + 8 * q);
+    } else {
+      const bf16* p = lds + (32 * ks + 8 * q + (c >> 2)) * PITCH + r16 + 4 * (c & 3);
+      return concat4(lds_read_tr16(p), lds_read_tr16(p + 4 * PITCH));
+    }
+  }
 };
 
 // Interior tiles with K a multiple of 64 take this kernel.  Same tiles and fragments as the
@@ -163,13 +174,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
                       (int64_t)kt0 * b_slab;
   const int64_t b_up = (int64_t)ep.I * ldb;   // from a gate row to its up row
 
-  f32x16 acc[WM][WN];
+  // The 16 x 16 x 32 instruction does the same work for less energy (a register-only loop sustains 12-14 % more with
+  // it at the package power limit); measured inside this kernel it is worth +3 % where both the main loop and the
+  // epilogue keep within the register file: 256 x 256 tiles, A contiguous along K, one pass over K, and not the
+  // SwiGLU epilogues.  Those instances run the main loop on 2 WM x 2 WN tiles of 16 x 16 and bring one band of
+  // accumulators at a time into the 32 x 32 layout that the epilogues are written for.
+  constexpr bool M16 = WM == 4 && WN == 4 && A_KC && !SPLITK && (EPI == EPI_NONE || EPI == EPI_RESIDUAL || EPI == EPI_ROPE);
+  f32x16 acc[M16 ? 1 : WM][M16 ? 1 : WN];
+  f32x4 acc16[M16 ? 2 * WM : 1][M16 ? 2 * WN : 1];
+  if constexpr (M16) {
 #pragma unroll
-  for (int a = 0; a < WM; a++)
+    for (int a = 0; a < 2 * WM; a++)
 #pragma unroll
-    for (int b = 0; b < WN; b++)
+      for (int b = 0; b < 2 * WN; b++) acc16[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  } else {
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+    for (int a = 0; a < WM; a++)
+#pragma unroll
+      for (int b = 0; b < WN; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
+  }
 
   bf16x8 ra[CA], rb[CB];
   auto gload_a = [&](int kt, int j) {
@@ -214,50 +239,131 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
   // the last k-step, behind its first group of MFMAs: by then every wavefront has written its part of slab
   // kt+1 and has read its last fragments of slab kt, so the fragments of slab kt+1's first k-step can be
   // fetched under the remaining MFMAs of slab kt instead of in front of an idle matrix pipe.
-  static_assert(CA == CB && KSTEPS > 1, "chunk schedule");
-  constexpr int MOVES = CA + CB, GROUPS = (KSTEPS - 1) * WM;
-  bf16x8 af[2][WM], bfr[2][WN];
-  if (nk > 0) {
+  if constexpr (M16) {
+    // The main loop on v_mfma_f32_16x16x32_bf16: 2 WM x 2 WN accumulator tiles of 16 x 16, two k-steps of 32 per slab;
+    // same LDS layout, same staging schedule.  The accumulators are brought into the 32 x 32 layout afterwards.
+    static_assert(CA == CB, "chunk schedule");
+    constexpr int WM2 = 2 * WM, WN2 = 2 * WN, KS2 = BK / 32;
+    static_assert(KS2 == 2 && WM2 == WN2, "fragment sets alternate per k-step");
+    constexpr int MOVES = CA + CB, GROUPS = (KS2 - 1) * WM2;
+    bf16x8 af[2][WM2], bfr[2][WN2];
+    if (nk > 0) {
 #pragma unroll
-    for (int a = 0; a < WM; a++) af[0][a] = TA::frag(As, 32 * (wm * WM + a), 0, g, i);
+      for (int a = 0; a < WM2; a++) af[0][a] = TA::frag16(As, 16 * (wm * WM2 + a), 0, lane);
 #pragma unroll
-    for (int b = 0; b < WN; b++) bfr[0][b] = TB::frag(Bs, 32 * (wn * WN + b), 0, g, i);
-  }
-  for (int kt = 0; kt < nk; kt++) {
-    const int buf = kt & 1;
-    const bf16* Ab = As + buf * TA::ELEMS;
-    const bf16* Bb = Bs + buf * TB::ELEMS;
-    const bf16* An = As + (buf ^ 1) * TA::ELEMS;
-    const bf16* Bn = Bs + (buf ^ 1) * TB::ELEMS;
-    const int kt2 = min(kt + 2, nk - 1);   // past the end: a harmless re-load, and a write nobody reads
-    GEMM_FENCE();
+      for (int b = 0; b < WN2; b++) bfr[0][b] = TB::frag16(Bs, 16 * (wn * WN2 + b), 0, lane);
+    }
+    for (int kt = 0; kt < nk; kt++) {
+      const int buf = kt & 1;
+      const bf16* Ab = As + buf * TA::ELEMS;
+      const bf16* Bb = Bs + buf * TB::ELEMS;
+      const bf16* An = As + (buf ^ 1) * TA::ELEMS;
+      const bf16* Bn = Bs + (buf ^ 1) * TB::ELEMS;
+      const int kt2 = min(kt + 2, nk - 1);   // past the end: a harmless re-load, and a write nobody reads
+      GEMM_FENCE();
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-      const int cur = ks & 1, nxt = cur ^ 1;
+      for (int ks = 0; ks < KS2; ks++) {
+        const int cur = ks & 1, nxt = cur ^ 1;
 #pragma unroll
-      for (int a = 0; a < WM; a++) {
+        for (int a = 0; a < WM2; a++) {
 #pragma unroll
-        for (int b = 0; b < WN; b++) acc[a][b] = mfma32(bfr[cur][b], af[cur][a], acc[a][b]);  // rows = n, cols = m
-        if (ks + 1 < KSTEPS) {
-          af[nxt][a] = TA::frag(Ab, 32 * (wm * WM + a), ks + 1, g, i);
-          if (a < WN) bfr[nxt][a] = TB::frag(Bb, 32 * (wn * WN + a), ks + 1, g, i);
-          const int gi = ks * WM + a;
+          for (int b = 0; b < WN2; b++)
+            acc16[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[cur][b], af[cur][a], acc16[a][b], 0, 0, 0);   // rows = n, cols = m
+          if (ks + 1 < KS2) {
+            af[nxt][a] = TA::frag16(Ab, 16 * (wm * WM2 + a), ks + 1, lane);
+            bfr[nxt][a] = TB::frag16(Bb, 16 * (wn * WN2 + a), ks + 1, lane);
+            const int gi = ks * WM2 + a;
 #pragma unroll
-          for (int m = gi * MOVES / GROUPS; m < (gi + 1) * MOVES / GROUPS; m++) {
-            if (m % 2 == 0) { sstore_a(buf ^ 1, m / 2); gload_a(kt2, m / 2); }
-            else { sstore_b(buf ^ 1, m / 2); gload_b(kt2, m / 2); }
+            for (int m = gi * MOVES / GROUPS; m < (gi + 1) * MOVES / GROUPS; m++) {
+              if (m % 2 == 0) { sstore_a(buf ^ 1, m / 2); gload_a(kt2, m / 2); }
+              else { sstore_b(buf ^ 1, m / 2); gload_b(kt2, m / 2); }
+            }
+          } else {
+            if (a == 0) __syncthreads();
+            af[nxt][a] = TA::frag16(An, 16 * (wm * WM2 + a), 0, lane);
+            bfr[nxt][a] = TB::frag16(Bn, 16 * (wn * WN2 + a), 0, lane);
           }
-        } else {
-          if (a == 0) __syncthreads();
-          // first fragments of the next slab (KSTEPS is even: they land in set 0)
-          af[nxt][a] = TA::frag(An, 32 * (wm * WM + a), 0, g, i);
-          if (a < WN) bfr[nxt][a] = TB::frag(Bn, 32 * (wn * WN + a), 0, g, i);
+          GEMM_FENCE();
         }
-        GEMM_FENCE();
+      }
+    }
+  } else {
+    static_assert(CA == CB && KSTEPS > 1, "chunk schedule");
+    constexpr int MOVES = CA + CB, GROUPS = (KSTEPS - 1) * WM;
+    bf16x8 af[2][WM], bfr[2][WN];
+    if (nk > 0) {
+#pragma unroll
+      for (int a = 0; a < WM; a++) af[0][a] = TA::frag(As, 32 * (wm * WM + a), 0, g, i);
+#pragma unroll
+      for (int b = 0; b < WN; b++) bfr[0][b] = TB::frag(Bs, 32 * (wn * WN + b), 0, g, i);
+    }
+    for (int kt = 0; kt < nk; kt++) {
+      const int buf = kt & 1;
+      const bf16* Ab = As + buf * TA::ELEMS;
+      const bf16* Bb = Bs + buf * TB::ELEMS;
+      const bf16* An = As + (buf ^ 1) * TA::ELEMS;
+      const bf16* Bn = Bs + (buf ^ 1) * TB::ELEMS;
+      const int kt2 = min(kt + 2, nk - 1);   // past the end: a harmless re-load, and a write nobody reads
+      GEMM_FENCE();
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+#pragma unroll
+        for (int a = 0; a < WM; a++) {
+#pragma unroll
+          for (int b = 0; b < WN; b++) acc[a][b] = mfma32(bfr[cur][b], af[cur][a], acc[a][b]);  // rows = n, cols = m
+          if (ks + 1 < KSTEPS) {
+            af[nxt][a] = TA::frag(Ab, 32 * (wm * WM + a), ks + 1, g, i);
+            if (a < WN) bfr[nxt][a] = TB::frag(Bb, 32 * (wn * WN + a), ks + 1, g, i);
+            const int gi = ks * WM + a;
+#pragma unroll
+            for (int m = gi * MOVES / GROUPS; m < (gi + 1) * MOVES / GROUPS; m++) {
+              if (m % 2 == 0) { sstore_a(buf ^ 1, m / 2); gload_a(kt2, m / 2); }
+              else { sstore_b(buf ^ 1, m / 2); gload_b(kt2, m / 2); }
+            }
+          } else {
+            if (a == 0) __syncthreads();
+            // first fragments of the next slab (KSTEPS is even: they land in set 0)
+            af[nxt][a] = TA::frag(An, 32 * (wm * WM + a), 0, g, i);
+            if (a < WN) bfr[nxt][a] = TB::frag(Bn, 32 * (wn * WN + a), 0, g, i);
+          }
+          GEMM_FENCE();
+        }
       }
     }
   }
-  __syncthreads();   // the epilogue reuses the operand buffers
+  __syncthreads();   // the epilogue (and the conversion in front of it) reuse the operand buffers
+  // lane l holds column m = l & 15 and rows n = 4 (l >> 4) + r of each 16 x 16 tile; the epilogues expect column
+  // m = l & 31 and rows n = 8 (r / 4) + 4 (l >> 5) + r % 4 of each 32 x 32 tile.  One band of WN tiles at a time
+  // makes a round trip through a private fp32 patch (a wavefront's LDS operations complete in order).
+  constexpr int CP = 36;
+  float* conv = reinterpret_cast<float*>(smem_raw) + 4 * 32 * (32 * WN + 4) + wave * 32 * CP;
+  static_assert(!M16 || (4 * 32 * (32 * WN + 4) + 4 * 32 * CP) * 4 <= 2 * (TA::ELEMS + TB::ELEMS) * 2, "the patches fit behind the bands");
+  f32x16 acc_row[WN];
+  auto load_row = [&](int a) {
+    if constexpr (!M16) return;
+    const int c = lane & 15, q4 = lane >> 4;
+#pragma unroll
+    for (int b = 0; b < WN; b++) {
+#pragma unroll
+      for (int ta = 0; ta < 2; ta++)
+#pragma unroll
+        for (int tb = 0; tb < 2; tb++)
+          *reinterpret_cast<f32x4*>(conv + (16 * ta + c) * CP + 16 * tb + 4 * q4) = acc16[2 * a + ta][2 * b + tb];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(conv + i * CP + 8 * q + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc_row[b][4 * q + e] = v[e];
+      }
+    }
+  };
+  auto acc_tile = [&](int a, int b) -> const f32x16& {
+    if constexpr (M16) return acc_row[b];
+    else return acc[a][b];
+  };
+#define ACC(a, b) acc_tile(a, b)
+#define LOAD_ROW(a) load_row(a)
 
   // Epilogue.  Lane (g, i) holds column m = i and rows n = 8*(r/4) + 4g + r%4 of each 32 x 32 tile,
   // i.e. 8-byte pieces of 32 different rows of C.  Unless C is accumulated into, the tiles go
@@ -270,13 +376,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     float* dst0 = part + ((int64_t)blockIdx.y * M + m0) * N + n0 + 32 * wn * WN;
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
 #pragma unroll
       for (int b = 0; b < WN; b++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           f32x4 v;
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          for (int e = 0; e < 4; e++) v[e] = ACC(a, b)[4 * q + e];
           *reinterpret_cast<f32x4*>(band + i * EPF + 32 * b + 8 * q + 4 * g) = v;
         }
       constexpr int CPR = 32 * WN / 4, RPP = 64 / CPR;                  // 16-byte chunks per row, rows per pass
@@ -296,13 +403,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     static_assert(4 * 32 * EPF * 2 <= 2 * (TA::ELEMS + TB::ELEMS), "the fp32 bands fit in the operand buffers");
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
 #pragma unroll
       for (int b = 0; b < WN; b++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           f32x4 v;
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          for (int e = 0; e < 4; e++) v[e] = ACC(a, b)[4 * q + e];
           *reinterpret_cast<f32x4*>(band + i * EPF + 32 * b + 8 * q + 4 * g) = v;
         }
       constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
@@ -327,13 +435,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     const int j0 = n0 / 2;   // first j of the tile
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
       bf16x4 gu[WN][4];
 #pragma unroll
       for (int b = 0; b < WN; b++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
 #pragma unroll
-          for (int e = 0; e < 4; e++) gu[b][q][e] = (bf16)acc[a][b][4 * q + e];
+          for (int e = 0; e < 4; e++) gu[b][q][e] = (bf16)ACC(a, b)[4 * q + e];
           *reinterpret_cast<bf16x4*>(band + i * EP + 32 * b + 8 * q + 4 * g) = gu[b][q];
         }
       constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
@@ -376,6 +485,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     const bool rotate = n0 + 32 * wn * WN < ep.I;   // this wavefront's head is a query or key head
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
       const int mrow = m0 + 32 * (wm * WM + a) + i;   // the token this lane holds
 #pragma unroll
       for (int bb = 0; bb < 2; bb++)
@@ -388,13 +498,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
 #pragma unroll
             for (int e = 0; e < 4; e++) {
               const float c = (float)cs[2 * e], sn = (float)cs[2 * e + 1];
-              const float x1 = acc[a][bb][4 * q + e], x2 = acc[a][bb + 2][4 * q + e];
+              const float x1 = ACC(a, bb)[4 * q + e], x2 = ACC(a, bb + 2)[4 * q + e];
               w1[e] = (bf16)(x1 * c - x2 * sn);
               w2[e] = (bf16)(x2 * c + x1 * sn);
             }
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) w1[e] = (bf16)acc[a][bb][4 * q + e], w2[e] = (bf16)acc[a][bb + 2][4 * q + e];
+            for (int e = 0; e < 4; e++) w1[e] = (bf16)ACC(a, bb)[4 * q + e], w2[e] = (bf16)ACC(a, bb + 2)[4 * q + e];
           }
           *reinterpret_cast<bf16x4*>(band + i * EP + 32 * bb + 8 * q + 4 * g) = w1;
           *reinterpret_cast<bf16x4*>(band + i * EP + 32 * (bb + 2) + 8 * q + 4 * g) = w2;
@@ -415,13 +525,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     bf16* band = reinterpret_cast<bf16*>(smem_raw) + wave * 32 * EP;
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
 #pragma unroll
       for (int b = 0; b < WN; b++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           bf16x4 w;
 #pragma unroll
-          for (int e = 0; e < 4; e++) w[e] = (bf16)acc[a][b][4 * q + e];
+          for (int e = 0; e < 4; e++) w[e] = (bf16)ACC(a, b)[4 * q + e];
           *reinterpret_cast<bf16x4*>(band + i * EP + 32 * b + 8 * q + 4 * g) = w;
         }
       constexpr int CPR = 32 * WN / 8, RPP = 64 / CPR;
@@ -452,6 +563,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     static_assert(4 * 32 * EP <= 2 * (TA::ELEMS + TB::ELEMS), "the bands fit in the operand buffers");
 #pragma unroll
     for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
 #pragma unroll
       for (int b = 0; b < WN; b++)
 #pragma unroll
@@ -459,7 +571,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
           const int nl = 32 * b + 8 * q + 4 * g;
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+          for (int e = 0; e < 4; e++) v[e] = ACC(a, b)[4 * q + e];
           if (bias) {
             const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n0 + 32 * wn * WN + nl);
 #pragma unroll
@@ -484,6 +596,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
   }
 #pragma unroll
   for (int a = 0; a < WM; a++) {
+    LOAD_ROW(a);
     const int m = m0 + 32 * (wm * WM + a) + i;
 #pragma unroll
     for (int b = 0; b < WN; b++) {
@@ -493,7 +606,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
         bf16* dst = C + (int64_t)m * ldc + n;
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = acc[a][b][4 * q + e];
+        for (int e = 0; e < 4; e++) v[e] = ACC(a, b)[4 * q + e];
         if (bias) {
           const bf16x4 bv = *reinterpret_cast<const bf16x4*>(bias + n);
 #pragma unroll
@@ -512,6 +625,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_fast_kernel(const bf16* __restr
     }
   }
 }
+
+#undef ACC
+#undef LOAD_ROW
 
 template <int WM, int WN, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
