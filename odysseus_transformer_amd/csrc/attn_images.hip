@@ -11,11 +11,7 @@ using namespace tile128;
 // an image leaves by a streaming store: this kernel does not read it again
 __device__ __forceinline__ void store_image_chunk(bf16* p, bf16x8 v) {
   typedef unsigned raw_t __attribute__((ext_vector_type(4)));
-#ifdef ODY_PLAIN_STORES
-  *reinterpret_cast<bf16x8*>(p) = v;
-#else
   __builtin_nontemporal_store(__builtin_bit_cast(raw_t, v), reinterpret_cast<raw_t*>(p));
-#endif
 }
 
 __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict__ src, AttnStrides s, int L,

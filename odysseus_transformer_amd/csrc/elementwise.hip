@@ -34,11 +34,7 @@ template <typename T> struct VecIO {
     vec_t v;
 #pragma unroll
     for (int e = 0; e < N; e++) v[e] = (T)f[e];
-#ifdef ODY_PLAIN_STORES
-    *reinterpret_cast<vec_t*>(p) = v;
-#else
     __builtin_nontemporal_store(__builtin_bit_cast(raw_t, v), reinterpret_cast<raw_t*>(p));
-#endif
   }
 };
 
