@@ -348,6 +348,18 @@ def main():
         kernels[name] = {"launches": n, "avg_ms": round(avg, 4), "min_ms": round(min_ms, 4)}
         if name in algo:
             kernels[name]["tflops"] = round(algo[name] / (avg * 1e-3) / 1e12, 1)
+        if name in ("attn_images", "attn_bwd_prepass"):
+            # memory-bound passes: algorithmic bytes (one 64-row image pass reads and writes L*H*D bf16; the
+            # query-side pre-pass reads Q, dO, O and lse and writes two images, delta and the start values)
+            # against the HBM peak and against a device copy that moves the same number of bytes
+            e = 2
+            nbytes = 2 * L * H * D * e if name == "attn_images" else (3 + 2) * L * H * D * e + 2 * L * H * 4 + (L // 64) * H * 1024
+            src = torch.empty(nbytes // 2, dtype=torch.uint8, device=dev)
+            dst = torch.empty_like(src)
+            ty = spread(time_events(lambda: dst.copy_(src), 20, 3))["median"]
+            del src, dst
+            kernels[name].update({"algorithmic_bytes": nbytes, "frac_of_hbm_peak": round(nbytes / (avg * 1e-3) / 1e9 / PEAK_HBM_GBS, 3),
+                                  "copy_yardstick_ms": round(ty, 4), "ours_over_yardstick": round(ty / avg, 3)})
         if name == "attn_bwd_dq_kept":   # bound by HBM: the kept dS, read once
             ds_bytes = _lib.load().ody_attn_bwd_ds_bytes(1, L, L, H, HKV, D, _lib.ODY_BF16, 1)
             kernels[name]["hbm_read_gbps"] = round(ds_bytes / (avg * 1e-3) / 1e9, 1)

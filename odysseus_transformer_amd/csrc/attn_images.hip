@@ -14,6 +14,19 @@ __device__ __forceinline__ void store_image_chunk(bf16* p, bf16x8 v) {
   __builtin_nontemporal_store(__builtin_bit_cast(raw_t, v), reinterpret_cast<raw_t*>(p));
 }
 
+// 16-byte chunk q of a tile's image, from the row-major copy of the tile in LDS (pitch 128 + 8): column
+// d = 16 (q >> 7) + (q & 15), and with c = (q >> 4) & 7 the rows 32 (e >> 2) + 4 (e & 3) + r0, e = 0..7, where
+// r0 = 16 (c & 1) + ((c >> 1) & 1) + 2 (c >> 2).  The 16 lanes of a transposing LDS read share c and the 16-column
+// block: lane 4 k + m points at row r0 + 4 k, columns 4 m .. 4 m + 3 of the block, and receives rows r0 + 4 k',
+// k' = 0..3, of column (its lane & 15) -- half a chunk per read instead of one element.
+__device__ __forceinline__ bf16x8 image_chunk(const bf16* tile, int q) {
+  constexpr int PITCH = 128 + 8;
+  const int c = (q >> 4) & 7, l = q & 15;
+  const int r0 = 16 * (c & 1) + ((c >> 1) & 1) + 2 * (c >> 2);
+  const bf16* p = tile + (r0 + 4 * (l >> 2)) * PITCH + 16 * (q >> 7) + 4 * (l & 3);
+  return concat4(lds_read_tr16(p), lds_read_tr16(p + 32 * PITCH));
+}
+
 __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict__ src, AttnStrides s, int L,
                                                           bf16* __restrict__ dst, int ntiles, int H,
                                                           int* __restrict__ flags, int nflags) {
@@ -35,16 +48,7 @@ __global__ __launch_bounds__(256) void attn_images_kernel(const bf16* __restrict
   bf16* img = dst + (((int64_t)b * H + h) * ntiles + t) * IMG_ELEMS;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
-    const int q = tid + 256 * j;                    // 16-byte chunk of the image
-    const int d = 16 * (q >> 7) + (q & 15), c = (q >> 4) & 7;
-    const int kt = c >> 2, ss = (c >> 1) & 1, g = c & 1;
-    bf16x8 v;
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      const int row = 32 * (e >> 2) + 16 * g + 4 * (e & 3) + ss + 2 * kt;
-      v[e] = tile[row * PITCH + d];
-    }
-    store_image_chunk(img + q * 8, v);
+    store_image_chunk(img + (tid + 256 * j) * 8, image_chunk(tile, tid + 256 * j));
   }
 }
 
@@ -93,16 +97,7 @@ __global__ __launch_bounds__(256) void attn_bwd_prepass_kernel(const AttnParams 
     bf16* img = (which ? doimg : qimg) + tile_id * IMG_ELEMS;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const int q = tid + 256 * j;                    // 16-byte chunk of the image
-      const int d = 16 * (q >> 7) + (q & 15), c = (q >> 4) & 7;
-      const int kt = c >> 2, ss = (c >> 1) & 1, g = c & 1;
-      bf16x8 v;
-#pragma unroll
-      for (int e = 0; e < 8; e++) {
-        const int row = 32 * (e >> 2) + 16 * g + 4 * (e & 3) + ss + 2 * kt;
-        v[e] = tile[row * PITCH + d];
-      }
-      store_image_chunk(img + q * 8, v);
+      store_image_chunk(img + (tid + 256 * j) * 8, image_chunk(tile, tid + 256 * j));
     }
   }
   if (tid < 128) {

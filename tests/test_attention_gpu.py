@@ -180,6 +180,28 @@ def test_attention_random_shapes(case, dev):
     assert_parity(dv, dv_ref, TOL_BF16, "dv")
 
 
+def _random_long_cases(n, seed):
+    """One long and one arbitrary side: the shapes on which the kernels cut a block's range into parts."""
+    g = torch.Generator().manual_seed(seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    cases = []
+    for _ in range(n):
+        hkv = [1, 2][r(0, 1)]
+        grp = [1, 2][r(0, 1)]
+        long, short = r(2049, 5200), r(1, 1400)
+        kind = r(0, 3)                       # 0: long queries, 1: long keys, 2: both long and causal, 3: causal with more keys
+        lq, lk = [(long, short), (short, long), (long, long), (short, short + long)][kind]
+        cases.append((1, lq, lk, hkv * grp, hkv, kind >= 2))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_long_cases(10, 31), ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d" % c)
+def test_attention_random_long_shapes(case, dev):
+    """Ragged lengths where one side is long enough for the key split of the forward and the range parts of the
+    backward to apply (recomputing kernels: the lengths are not multiples of 256)."""
+    test_attention_random_shapes(case, dev)
+
+
 @pytest.mark.parametrize("D", [64, 128])
 @pytest.mark.parametrize("case", _random_cases(10, 77), ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_c%d" % c)
 def test_attention_random_shapes_fp32(case, D, dev):
