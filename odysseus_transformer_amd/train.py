@@ -140,6 +140,9 @@ def main(args) -> dict:
     from . import _lib
 
     assert args.batch_size == 1, "Only support batch size 1"
+    if getattr(args, "cpu_offload", False):
+        raise NotImplementedError("--cpu-offload is FSDP's parameter offload (train.py:123-157 of the reference); "
+                                  "the FSDP wrapping is outside this build")
     rank, world_size = 0, 1
     _lib.load()
     torch.manual_seed(args.seed)
@@ -248,6 +251,12 @@ def parse_args(argv=None):
     ap.add_argument("--seq-length", type=int, default=16384)
     ap.add_argument("--grad-checkpoint", action="store_true", default=False,
                     help="drop every decoder layer's activations after the forward pass and recompute them in backward")
+    ap.add_argument("--cpu-offload", action="store_true", default=False,
+                    help="accepted for command-line compatibility (train.py:252 of the reference): FSDP's parameter "
+                         "offload to the host is part of the FSDP wrapping, which is outside this build; refused")
+    ap.add_argument("--use_zero2", action="store_true", default=False,
+                    help="accepted for command-line compatibility (train.py:254): FSDP's SHARD_GRAD_OP strategy; with one "
+                         "rank there is nothing to shard, so it changes nothing here")
     ap.add_argument("--use_ody_zero3", action="store_true", default=True)
     ap.add_argument("--use_profiler", action="store_true", default=False,
                     help="torch.profiler over steps 2-5 (two warm-up, four recorded), trace under ./profile/")

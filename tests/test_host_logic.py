@@ -323,6 +323,15 @@ def test_train_script_accepts_every_mode_of_the_reference():
     from odysseus_transformer_amd.train import parse_args
     for mode in ("odysseus", "ulysses", "dp", "tpsp", "ring"):
         assert parse_args(["--parallel_mode", mode]).parallel_mode == mode
+    # every flag of the reference's parser (train.py:245-257) is accepted; the FSDP ones say what they do here
+    ref_flags = ["--batch-size", "1", "--seed", "1", "--max-train-steps", "3", "--learning-rate", "1e-5", "--rope-theta", "1e4",
+                 "--model", "x", "--seq-length", "1024", "--cpu-offload", "--grad-checkpoint", "--use_zero2", "--use_ody_zero3",
+                 "--use_profiler", "--use_cfg_init_model"]
+    a = parse_args(ref_flags)
+    assert a.cpu_offload and a.use_zero2 and a.grad_checkpoint and a.use_profiler and a.seq_length == 1024
+    from odysseus_transformer_amd.train import main
+    with pytest.raises(NotImplementedError, match="cpu-offload"):
+        main(a)
 
 
 def test_adamw_host_side():
