@@ -309,6 +309,40 @@ int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o
                       void* workspace, size_t workspace_bytes, void* stream,
                       const void* rope_table_q, const void* rope_table_k);
 
+/* ---- attention dropout ------------------------------------------------------
+ * The dropout_p argument of the attention routine the reference calls (decoder/odysseus.py:228, 256-263; it
+ * passes config.attention_dropout while training, 0.0 in its own configurations).  ody_attn_fwd / ody_attn_bwd with
+ * two more arguments: an entry of the softmax matrix P is dropped with probability p_drop before P . V and the
+ * kept entries are scaled by 1 / (1 - p_drop); lse is that of the full P.  Which entries are dropped is a fixed
+ * function of (seed, batch, query head, query, key) -- a 32-bit counter hash, restated on the host in
+ * oracle/odysseus_oracle.py -- so the backward reproduces the forward's mask from the same seed.  The reference's
+ * routine draws its mask from a Philox stream of its own: masks differ, the distribution and the arithmetic given a
+ * mask are the same.  bf16 only, head_dim 64 or 128, on the library's plain kernels (no key split, no kept dS, no
+ * rotary tables: ODY_BWD_KEEP_DS is refused); p_drop = 0 is exactly ody_attn_fwd / ody_attn_bwd.  Workspaces as
+ * for those.
+ */
+int ody_attn_fwd_dropout(const void* q, const void* k, const void* v, void* out, float* lse,
+                         int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                         int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                         int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                         int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                         int64_t so_b, int64_t so_l, int64_t so_h,
+                         float scale, int causal, int dtype,
+                         void* workspace, size_t workspace_bytes, void* stream, float p_drop, uint64_t seed);
+int ody_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                         const void* dout, void* dq, void* dk, void* dv,
+                         int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                         int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                         int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                         int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                         int64_t so_b, int64_t so_l, int64_t so_h,
+                         int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                         int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                         int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                         int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                         float scale, int causal, int flags, int dtype,
+                         void* workspace, size_t workspace_bytes, void* stream, float p_drop, uint64_t seed);
+
 /* ---- optimizer ------------------------------------------------------------
  * One step of torch.optim.AdamW (the optimizer of the reference's training loop, train.py:170,216) on one
  * tensor of n elements, in one pass instead of the host framework's seven element-wise passes:

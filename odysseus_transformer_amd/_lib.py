@@ -16,7 +16,7 @@ GEMM_NT, GEMM_NN, GEMM_TN = 0, 1, 2
 BWD_ACCUMULATE_DQ, BWD_DQ_F32, BWD_REUSE_QUERY_SIDE, BWD_KEEP_DS = 1, 2, 4, 8
 ATTN_FWD_NOALLOC_SCRATCH_BYTES = (32 << 20) + (64 << 10)
 
-_i, _i64, _f, _p, _sz = C.c_int, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
+_i, _i64, _u64, _f, _p, _sz = C.c_int, C.c_int64, C.c_uint64, C.c_float, C.c_void_p, C.c_size_t
 
 # name -> (restype, argtypes); mirrors include/odysseus_hip.h one to one
 SIGNATURES = {
@@ -51,6 +51,8 @@ SIGNATURES = {
     "ody_adamw": (_i, [_p, _p, _p, _p, _i64, _f, _f, _f, _f, _f, _i64, _i, _p]),
     "ody_linear_rope": (_i, [_p] * 4 + [_i] * 5 + [_i64] * 4 + [_i, _p]),
     "ody_attn_bwd_rope": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p, _p, _p]),
+    "ody_attn_fwd_dropout": (_i, [_p] * 5 + [_i] * 6 + [_i64] * 12 + [_f, _i, _i, _p, _sz, _p, _f, _u64]),
+    "ody_attn_bwd_dropout": (_i, [_p] * 9 + [_i] * 6 + [_i64] * 24 + [_f, _i, _i, _i, _p, _sz, _p, _f, _u64]),
 }
 
 _lib = None

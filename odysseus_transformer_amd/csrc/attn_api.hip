@@ -36,6 +36,60 @@ int check_tensor(const char* who, const char* name, const void* ptr, const AttnS
 
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 
+namespace {
+// p_drop in (0, 1): the dropout fields of the argument block; 0: none.  bf16 only (the kernels that implement it).
+int set_dropout(const char* who, AttnParams& p, float p_drop, uint64_t seed, int dtype) {
+  ODY_REQUIRE(p_drop >= 0.f && p_drop < 1.f, ODY_ERR_BAD_SHAPE, "%s: the dropout probability must be in [0, 1), got %g", who,
+              (double)p_drop);
+  if (p_drop == 0.f) return ODY_OK;
+  ODY_REQUIRE(dtype == ODY_BF16, ODY_ERR_UNSUPPORTED, "%s: attention dropout is implemented for bf16 only", who);
+  const double t = (double)p_drop * 4294967296.0;
+  p.drop_thresh = t >= 4294967295.0 ? 4294967295u : (t < 1.0 ? 1u : (unsigned)t);
+  p.drop_seed = (unsigned)(seed ^ (seed >> 32));
+  p.drop_scale = 1.f / (1.f - p_drop);
+  return ODY_OK;
+}
+
+int attn_fwd_impl(const char* who, const void* q, const void* k, const void* v, void* out, float* lse,
+                  int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                  int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                  int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                  int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                  int64_t so_b, int64_t so_l, int64_t so_h,
+                  float scale, int causal, int dtype, void* workspace, size_t workspace_bytes,
+                  void* stream, float p_drop, uint64_t seed) {
+  int rc = check_common(who, B, Lq, Lk, Hq, Hkv, D, dtype);
+  if (rc) return rc;
+  AttnParams p{};
+  if ((rc = set_dropout(who, p, p_drop, seed, dtype))) return rc;
+  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
+  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
+  p.causal = causal ? 1 : 0; p.off = Lk - Lq;
+  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
+  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
+  const bool vec = true;
+  if ((rc = check_tensor(who, "q", q, p.sq, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "k", k, p.sk, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "v", v, p.sv, dtype, vec))) return rc;
+  if ((rc = check_tensor(who, "out", out, p.so, dtype, vec))) return rc;
+  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "%s: lse is NULL", who);
+  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "%s: scale must be positive", who);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == ODY_BF16 && D == 128 && p.drop_thresh == 0) {
+    // the least that will do: without room for the parts of a key-split call the call runs unsplit
+    const size_t need = (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255;
+    ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "%s: workspace is NULL", who);
+    ODY_REQUIRE(workspace_bytes >= need, ODY_ERR_WORKSPACE, "%s: workspace of %zu bytes, %zu needed", who,
+                workspace_bytes, need);
+    ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
+                "%s: workspace must be 256-byte aligned", who);
+    return ody_launch_attn_fwd_w8(p, workspace, workspace_bytes, st);
+  }
+  if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
+  return ody_launch_attn_fwd_f32(p, D, st);
+}
+}  // namespace
+
 extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
                             int B, int Lq, int Lk, int Hq, int Hkv, int D,
                             int64_t sq_b, int64_t sq_l, int64_t sq_h,
@@ -44,34 +98,20 @@ extern "C" int ody_attn_fwd(const void* q, const void* k, const void* v, void* o
                             int64_t so_b, int64_t so_l, int64_t so_h,
                             float scale, int causal, int dtype, void* workspace, size_t workspace_bytes,
                             void* stream) {
-  int rc = check_common("ody_attn_fwd", B, Lq, Lk, Hq, Hkv, D, dtype);
-  if (rc) return rc;
-  AttnParams p{};
-  p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
-  p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
-  p.causal = causal ? 1 : 0; p.off = Lk - Lq;
-  p.scale = scale; p.scale_log2e = scale * ODY_LOG2E;
-  p.sq = {sq_b, sq_l, sq_h}; p.sk = {sk_b, sk_l, sk_h}; p.sv = {sv_b, sv_l, sv_h}; p.so = {so_b, so_l, so_h};
-  const bool vec = true;
-  if ((rc = check_tensor("ody_attn_fwd", "q", q, p.sq, dtype, vec))) return rc;
-  if ((rc = check_tensor("ody_attn_fwd", "k", k, p.sk, dtype, vec))) return rc;
-  if ((rc = check_tensor("ody_attn_fwd", "v", v, p.sv, dtype, vec))) return rc;
-  if ((rc = check_tensor("ody_attn_fwd", "out", out, p.so, dtype, vec))) return rc;
-  ODY_REQUIRE(lse != nullptr, ODY_ERR_NULL, "ody_attn_fwd: lse is NULL");
-  ODY_REQUIRE(scale > 0.f && std::isfinite(scale), ODY_ERR_BAD_SHAPE, "ody_attn_fwd: scale must be positive");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == ODY_BF16 && D == 128) {
-    // the least that will do: without room for the parts of a key-split call the call runs unsplit
-    const size_t need = (ody_attn_fwd_w8_workspace(B, Lq, Lk, Hq, Hkv, false) + 255) & ~(size_t)255;
-    ODY_REQUIRE(workspace != nullptr, ODY_ERR_NULL, "ody_attn_fwd: workspace is NULL");
-    ODY_REQUIRE(workspace_bytes >= need, ODY_ERR_WORKSPACE, "ody_attn_fwd: workspace of %zu bytes, %zu needed",
-                workspace_bytes, need);
-    ODY_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, ODY_ERR_MISALIGNED,
-                "ody_attn_fwd: workspace must be 256-byte aligned");
-    return ody_launch_attn_fwd_w8(p, workspace, workspace_bytes, st);
-  }
-  if (dtype == ODY_BF16) return ody_launch_attn_fwd_mfma(p, D, st);
-  return ody_launch_attn_fwd_f32(p, D, st);
+  return attn_fwd_impl("ody_attn_fwd", q, k, v, out, lse, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h,
+                       so_b, so_l, so_h, scale, causal, dtype, workspace, workspace_bytes, stream, 0.f, 0);
+}
+
+extern "C" int ody_attn_fwd_dropout(const void* q, const void* k, const void* v, void* out, float* lse,
+                                    int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                                    int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                                    int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                                    int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                                    int64_t so_b, int64_t so_l, int64_t so_h,
+                                    float scale, int causal, int dtype, void* workspace, size_t workspace_bytes,
+                                    void* stream, float p_drop, uint64_t seed) {
+  return attn_fwd_impl("ody_attn_fwd_dropout", q, k, v, out, lse, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l,
+                       sv_h, so_b, so_l, so_h, scale, causal, dtype, workspace, workspace_bytes, stream, p_drop, seed);
 }
 
 namespace {
@@ -161,12 +201,16 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
                   int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
                   int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
                   float scale, int causal, int flags, int dtype,
-                  void* workspace, size_t workspace_bytes, void* stream) {
+                  void* workspace, size_t workspace_bytes, void* stream, float p_drop = 0.f, uint64_t seed = 0) {
   int rc = check_common(who, B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
   ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE | ODY_BWD_KEEP_DS)) == 0, ODY_ERR_UNSUPPORTED,
               "%s: unknown flag bits in %d", who, flags);
   AttnParams p{};
+  if ((rc = set_dropout(who, p, p_drop, seed, dtype))) return rc;
+  ODY_REQUIRE(p.drop_thresh == 0 || !(flags & ODY_BWD_KEEP_DS), ODY_ERR_UNSUPPORTED,
+              "%s: ODY_BWD_KEEP_DS is not available with dropout", who);
+  ODY_REQUIRE(p.drop_thresh == 0 || !(rope_q || rope_k), ODY_ERR_UNSUPPORTED, "%s: no rotary tables with dropout", who);
   p.q = q; p.k = k; p.v = v; p.out = const_cast<void*>(out); p.lse = const_cast<float*>(lse);
   p.dout = dout; p.dq = dq; p.dk = dk; p.dv = dv;
   p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
@@ -212,7 +256,7 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
   p.delta = static_cast<float*>(workspace);
   if (ws_ds) p.ds = reinterpret_cast<bf16*>(static_cast<char*>(workspace) + ws_base);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (dtype == ODY_BF16 && D == 128)   // its query-side pre-pass computes delta as well
+  if (dtype == ODY_BF16 && D == 128 && p.drop_thresh == 0)   // its query-side pre-pass computes delta as well
     return ody_launch_attn_bwd_pipe(p, static_cast<char*>(workspace) + delta_bytes(B, Lq, Hq), st);
   if (!p.reuse_query_side && (rc = ody_launch_attn_delta(p, D, dtype, st))) return rc;
   if (dtype == ODY_BF16) return ody_launch_attn_bwd_mfma(p, D, st);
@@ -236,6 +280,25 @@ extern "C" int ody_attn_bwd(const void* q, const void* k, const void* v, const v
   return attn_bwd_impl("ody_attn_bwd", nullptr, nullptr, q, k, v, out, lse, dout, dq, dk, dv, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l, sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h,
                        so_b, so_l, so_h, sdo_b, sdo_l, sdo_h, sdq_b, sdq_l, sdq_h, sdk_b, sdk_l, sdk_h, sdv_b, sdv_l, sdv_h, scale,
                        causal, flags, dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ody_attn_bwd_dropout(const void* q, const void* k, const void* v, const void* out, const float* lse,
+                                    const void* dout, void* dq, void* dk, void* dv,
+                                    int B, int Lq, int Lk, int Hq, int Hkv, int D,
+                                    int64_t sq_b, int64_t sq_l, int64_t sq_h,
+                                    int64_t sk_b, int64_t sk_l, int64_t sk_h,
+                                    int64_t sv_b, int64_t sv_l, int64_t sv_h,
+                                    int64_t so_b, int64_t so_l, int64_t so_h,
+                                    int64_t sdo_b, int64_t sdo_l, int64_t sdo_h,
+                                    int64_t sdq_b, int64_t sdq_l, int64_t sdq_h,
+                                    int64_t sdk_b, int64_t sdk_l, int64_t sdk_h,
+                                    int64_t sdv_b, int64_t sdv_l, int64_t sdv_h,
+                                    float scale, int causal, int flags, int dtype,
+                                    void* workspace, size_t workspace_bytes, void* stream, float p_drop, uint64_t seed) {
+  return attn_bwd_impl("ody_attn_bwd_dropout", nullptr, nullptr, q, k, v, out, lse, dout, dq, dk, dv, B, Lq, Lk, Hq, Hkv, D, sq_b, sq_l,
+                       sq_h, sk_b, sk_l, sk_h, sv_b, sv_l, sv_h, so_b, so_l, so_h, sdo_b, sdo_l, sdo_h, sdq_b, sdq_l, sdq_h, sdk_b,
+                       sdk_l, sdk_h, sdv_b, sdv_l, sdv_h, scale, causal, flags, dtype, workspace, workspace_bytes, stream, p_drop,
+                       seed);
 }
 
 extern "C" int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* out, const float* lse,

@@ -72,7 +72,9 @@ __device__ __forceinline__ bf16x8 lds_tr_frag(const bf16* tile, int row32, int s
 // ---------------------------------------------------------------------------
 // dK / dV
 // ---------------------------------------------------------------------------
-template <int D>
+// DROP (both kernels): attention dropout as the forward applied it (ody_dropout_hash): dV takes the kept entries of P
+// scaled by 1 / (1 - p), and dP = dO V^T counts only where the entry was kept, with the same scale.
+template <int D, bool DROP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams p) {
   constexpr int BQ = 64, WK = 32, BN = 4 * WK, P = D + 8, KS = D / 16, DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -147,6 +149,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 
   for (int it = 0; it < total; it++) {
     const int buf = it & 1;
+    const unsigned dh = DROP ? ody_dropout_head(p.drop_seed, b * p.Hq + hk * p.group + it / ntq) : 0u;
     const int i0 = i_begin + (ntq - 1 - it % ntq) * BQ;   // last query tile first: the key blocks running on an XCD then read the same Q / dO tiles together
     if (it + 1 < total) gload(it + 1);
     const bf16* Qb = Qs + buf * BQ * P;
@@ -179,8 +182,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams 
             const int qi = m0 + kap(rho_of(r, g));
             if (key > qi + p.off) pr = 0.f;
           }
-          const float dsv = pr * (dp[r] - d4[e]);
-          pf[r >> 3][r & 7] = (bf16)pr;
+          float dpv = dp[r], pv = pr;
+          if (DROP) {
+            const bool keep = ody_dropout_hash(ody_dropout_row(dh, m0 + kap(rho_of(r, g))), key) >= p.drop_thresh;
+            dpv = keep ? dpv * p.drop_scale : 0.f;
+            pv = keep ? pr : 0.f;
+          }
+          const float dsv = pr * (dpv - d4[e]);
+          pf[r >> 3][r & 7] = (bf16)pv;
           dsf[r >> 3][r & 7] = (bf16)dsv;
         }
       }
@@ -208,7 +217,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           wk[e] = (bf16)(dk[dt][4 * a + e] * p.scale);
-          wv[e] = (bf16)dv[dt][4 * a + e];
+          wv[e] = (bf16)(DROP ? dv[dt][4 * a + e] * p.drop_scale : dv[dt][4 * a + e]);
         }
         *reinterpret_cast<bf16x4*>(dkp + 32 * dt + 8 * a + 4 * g) = wk;
         *reinterpret_cast<bf16x4*>(dvp + 32 * dt + 8 * a + 4 * g) = wv;
@@ -219,7 +228,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkdv_kernel(const AttnParams 
 // ---------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
   constexpr int BN = 64, WQ = 32, BM = 4 * WQ, P = D + 8, KS = D / 16, DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -254,6 +263,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
   lse2 *= ODY_LOG2E;
   const float delta = (qi < p.Lq) ? p.delta[ri] : 0.f;
   const int lim = p.causal ? min(p.Lk - 1, qi + p.off) : p.Lk - 1;
+  const unsigned drow = DROP ? ody_dropout_row(ody_dropout_head(p.drop_seed, b * p.Hq + h), qi) : 0u;
 
   f32x16 dq[DT];
 #pragma unroll
@@ -306,7 +316,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
           const int kj = k0 + kap(rho_of(r, g));
           if (kj > lim) pr = 0.f;
         }
-        dsf[r >> 3][r & 7] = (bf16)(pr * (dp[r] - delta));
+        float dpv = dp[r];
+        if (DROP) dpv = ody_dropout_hash(drow, k0 + kap(rho_of(r, g))) >= p.drop_thresh ? dpv * p.drop_scale : 0.f;
+        dsf[r >> 3][r & 7] = (bf16)(pr * (dpv - delta));
       }
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
@@ -350,27 +362,32 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnParams p) {
   }
 }
 
-template <int D>
+template <int D, bool DROP>
 int launch(const AttnParams& p, hipStream_t st) {
   constexpr size_t smem_kv = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16) + 2 * 2 * 64 * sizeof(float);
   constexpr size_t smem_q = (size_t)2 * 2 * 64 * (D + 8) * sizeof(bf16);
-  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D>), smem_kv, "attn_bwd"))
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<D, DROP>), smem_kv, "attn_bwd"))
     return rc;
-  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D>), smem_q, "attn_bwd"))
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, DROP>), smem_q, "attn_bwd"))
     return rc;
   dim3 gk(((p.Lk + 127) / 128) * p.Hkv * p.B);
-  ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D>), gk, dim3(256), smem_kv, p);
+  ODY_LAUNCH("attn_bwd_dkdv", st, (attn_bwd_dkdv_kernel<D, DROP>), gk, dim3(256), smem_kv, p);
   int rc = ody_check_launch("attn_bwd_dkdv");
   if (rc) return rc;
   dim3 gq(((p.Lq + 127) / 128) * p.Hq * p.B);
-  ODY_LAUNCH("attn_bwd_dq", st, (attn_bwd_dq_kernel<D>), gq, dim3(256), smem_q, p);
+  ODY_LAUNCH("attn_bwd_dq", st, (attn_bwd_dq_kernel<D, DROP>), gq, dim3(256), smem_q, p);
   return ody_check_launch("attn_bwd_dq");
 }
 
 }  // namespace
 
 int ody_launch_attn_bwd_mfma(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 64) return launch<64>(p, st);   // head_dim 128 has its own kernels (attn_bwd_pipe.hip)
-  ody_set_error("attn_bwd: head_dim %d not built here (64)", D);
+  if (p.drop_thresh != 0) {   // dropout: these kernels serve both head dims
+    if (D == 64) return launch<64, true>(p, st);
+    if (D == 128) return launch<128, true>(p, st);
+  } else if (D == 64) {
+    return launch<64, false>(p, st);   // head_dim 128 has its own kernels (attn_bwd_pipe.hip)
+  }
+  ody_set_error("attn_bwd: head_dim %d not built here", D);
   return ODY_ERR_UNSUPPORTED;
 }

@@ -24,7 +24,9 @@
 
 namespace {
 
-template <int D, int QT>
+// DROP: attention dropout (AttnParams::drop_*): the row sums, and with them lse, are those of the full P; the entries
+// that go into P . V are the kept ones, and the result is scaled by 1 / (1 - p) at the end.
+template <int D, int QT, bool DROP>
 __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams p, const int* __restrict__ flags,
                                                                int flag_block) {
   constexpr int BN = 64, WQ = 32 * QT, BM = 4 * WQ;
@@ -113,6 +115,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams 
   __syncthreads();
 
   const float c2 = p.scale_log2e;
+  unsigned drow[QT];
+  if (DROP) {
+    const unsigned dh = ody_dropout_head(p.drop_seed, b * p.Hq + h);
+#pragma unroll
+    for (int qt = 0; qt < QT; qt++) drow[qt] = ody_dropout_row(dh, wq0 + 32 * qt + i);
+  }
   // transpose-read addressing inside a 16-lane block
   const int tr_row = (i & 15) >> 2, tr_col = 16 * (i >> 4) + 4 * (i & 3);
 
@@ -190,7 +198,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams 
 #pragma unroll
           for (int ss = 0; ss < 2; ss++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) pb[qt][kt][ss][e] = (bf16)s[qt][kt][8 * ss + e];
+            for (int e = 0; e < 8; e++) {
+              float x = s[qt][kt][8 * ss + e];
+              if (DROP) {
+                const int r = 8 * ss + e, key = n0 + 32 * kt + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (ody_dropout_hash(drow[qt], key) < p.drop_thresh) x = 0.f;
+              }
+              pb[qt][kt][ss][e] = (bf16)x;
+            }
       }
       // ---- O^T += V^T . P^T
 #pragma unroll
@@ -219,7 +234,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams 
   for (int qt = 0; qt < QT; qt++) {
     const int qi = wq0 + 32 * qt + i;
     const float lt = l[qt] + xor32(l[qt]);
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    const float inv = lt > 0.f ? (DROP ? p.drop_scale : 1.f) / lt : 0.f;
     if (qi < p.Lq) {
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
@@ -235,26 +250,31 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(const AttnParams 
   }
 }
 
-template <int D, int QT>
+template <int D, int QT, bool DROP>
 int launch(const AttnParams& p, const int* flags, int flag_block, hipStream_t st) {
   constexpr int BN = 64, BM = 4 * 32 * QT;
   constexpr size_t smem = (size_t)2 * BN * ((D + 8) + (D + 32)) * sizeof(bf16);
-  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_fwd_mfma_kernel<D, QT>), smem, "attn_fwd"))
+  if (int rc = ody_allow_dynamic_lds(reinterpret_cast<const void*>(&attn_fwd_mfma_kernel<D, QT, DROP>), smem, "attn_fwd"))
     return rc;
   dim3 grid(((p.Lq + BM - 1) / BM) * p.Hq * p.B);
-  ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT>), grid, dim3(256), smem, p, flags, flag_block);
+  ODY_LAUNCH("attn_fwd_mfma", st, (attn_fwd_mfma_kernel<D, QT, DROP>), grid, dim3(256), smem, p, flags, flag_block);
   return ody_check_launch("attn_fwd_mfma");
 }
 
 }  // namespace
 
 int ody_launch_attn_fwd_mfma(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 128) return launch<128, 1>(p, nullptr, 1, st);
-  if (D == 64) return launch<64, 1>(p, nullptr, 1, st);
+  if (p.drop_thresh != 0) {
+    if (D == 128) return launch<128, 1, true>(p, nullptr, 1, st);
+    if (D == 64) return launch<64, 1, true>(p, nullptr, 1, st);
+  } else {
+    if (D == 128) return launch<128, 1, false>(p, nullptr, 1, st);
+    if (D == 64) return launch<64, 1, false>(p, nullptr, 1, st);
+  }
   ody_set_error("attn_fwd: head_dim %d not built (64, 128)", D);
   return ODY_ERR_UNSUPPORTED;
 }
 
 int ody_launch_attn_fwd_mfma_flagged(const AttnParams& p, const int* flags, int block, hipStream_t st) {
-  return launch<128, 1>(p, flags, block, st);
+  return launch<128, 1, false>(p, flags, block, st);
 }

@@ -31,6 +31,11 @@ struct AttnParams {
   // bwd, bf16 head_dim 128, Lq and Lk multiples of 256 (causal: Lq == Lk): when set, the dK/dV kernel keeps
   // every dS tile here (ody_attn_bwd_ds_bytes) and dQ is computed from them instead of from a second pass over S and dP
   bf16* ds;
+  // attention dropout (bf16, the kernels of attn_fwd_mfma.hip / attn_bwd_mfma.hip only): an entry of P is dropped when
+  // its 32-bit hash (ody_dropout_hash) is below drop_thresh = p * 2^32; kept entries are scaled by drop_scale =
+  // 1 / (1 - p).  drop_thresh == 0: no dropout.
+  unsigned drop_thresh, drop_seed;
+  float drop_scale;
   float scale;        // softmax scale
   float scale_log2e;  // scale * log2(e)
   AttnStrides sq, sk, sv, so, sdo, sdq, sdk, sdv;
@@ -50,6 +55,20 @@ __device__ __forceinline__ BlockCoord ody_block_coord_of(int id, int H, int B) {
   return BlockCoord{id / (H * B), hb % H, hb / H};
 }
 __device__ __forceinline__ BlockCoord ody_block_coord(int H, int B) { return ody_block_coord_of(blockIdx.x, H, B); }
+
+// The dropout decision of score (batch b, query head h, query q, key k): a counter-based hash, so that the forward
+// kernel and both backward kernels, which hold the scores in different layouts, agree without exchanging anything.
+//   head value  u = mix(seed ^ (b * Hq + h) * 0x85ebca77)        (once per block)
+//   row value   r = mix(u + q * 0x9e3779b1)                      (once per query)
+//   hash        x = mix(r ^ k * 0xc2b2ae3d);  the score is kept iff x >= thresh
+// mix is the 32-bit finalizer of MurmurHash3.  tests/ restate it in integer arithmetic on the host.
+__device__ __forceinline__ unsigned ody_mix32(unsigned x) {
+  x ^= x >> 16; x *= 0x85ebca6bu; x ^= x >> 13; x *= 0xc2b2ae35u; x ^= x >> 16;
+  return x;
+}
+__device__ __forceinline__ unsigned ody_dropout_head(unsigned seed, int bh) { return ody_mix32(seed ^ ((unsigned)bh * 0x85ebca77u)); }
+__device__ __forceinline__ unsigned ody_dropout_row(unsigned head, int q) { return ody_mix32(head + (unsigned)q * 0x9e3779b1u); }
+__device__ __forceinline__ unsigned ody_dropout_hash(unsigned row, int k) { return ody_mix32(row ^ ((unsigned)k * 0xc2b2ae3du)); }
 #endif
 
 // Launchers (one per translation unit); each returns an ody_status.

@@ -145,9 +145,8 @@ class LlamaFlashAttention2TPSP(nn.Module):
         # the training path: no padding and nothing in the cache yet.  A padding mask or earlier cache content takes
         # the general path below, as decoder/odysseus.py:215-263 hands both on to the host's flash-attention call.
         cached = past_key_value is not None and past_key_value.get_seq_length(self.layer_idx) > 0
-        general = cached or attention_mask is not None
-        if self.training and self.attention_dropout != 0.0:
-            raise NotImplementedError("attention dropout is not implemented (the reference trains with 0.0)")
+        dropout = self.attention_dropout if self.training else 0.0   # decoder/odysseus.py:228
+        general = cached or attention_mask is not None or dropout != 0.0
         scale = 1.0 / math.sqrt(self.head_dim)
         nh, nkv, D = self.n_local_heads, self.n_local_kv_heads, self.head_dim
 
@@ -159,7 +158,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
                 qkv = self.qkv_proj(hidden_states).view(bsz, q_len, nh + 2 * nkv, D)
                 qkv = ops.apply_rope_packed(qkv, nh + nkv, position_ids, self.rope_theta)
                 attn_output = self._attend_general(qkv[:, :, :nh], qkv[:, :, nh:nh + nkv], qkv[:, :, nh + nkv:],
-                                                   attention_mask, past_key_value, cache_position, scale)
+                                                   attention_mask, past_key_value, cache_position, scale, dropout)
             elif self._can_fuse_rope(hidden_states):
                 # projection, rotary embedding and attention as one autograd node: the rotation rides in the
                 # projection's epilogue, its backward in the epilogues of the attention backward
@@ -180,7 +179,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
             q = ops.apply_rope_packed(q, nh, position_ids, self.rope_theta)
             k = ops.apply_rope_packed(k, nkv, position_ids, self.rope_theta)
             if general:
-                attn_output = self._attend_general(q, k, v, attention_mask, past_key_value, cache_position, scale)
+                attn_output = self._attend_general(q, k, v, attention_mask, past_key_value, cache_position, scale, dropout)
             else:
                 if past_key_value is not None:
                     self._update_cache(past_key_value, k.detach(), v.detach(), q_len, cache_position)
@@ -225,7 +224,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
                                 {"cache_position": cache_position})
         assert k_all.shape[-2] == q_len, "the cache was not empty"
 
-    def _attend_general(self, q, k, v, attention_mask, cache, cache_position, scale):
+    def _attend_general(self, q, k, v, attention_mask, cache, cache_position, scale, dropout=0.0):
         """Attention of the rotated q (1, Lq, nh, D) over k, v (1, Lq, nkv, D) appended to the cache's earlier
         content, with an optional padding mask (1, Lk) of 0 / 1 over all keys -- what decoder/odysseus.py:215-263
         reaches through the cache's update() and the host's flash-attention forward: queries sit at the END of
@@ -238,7 +237,7 @@ class LlamaFlashAttention2TPSP(nn.Module):
             k, v = k_all.transpose(1, 2), v_all.transpose(1, 2)
         Lq, Lk = q.shape[1], k.shape[1]
         if attention_mask is None:
-            return ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+            return ops.flash_attn_func(q, k, v, dropout, softmax_scale=scale, causal=True)
         if attention_mask.dim() != 2 or attention_mask.shape[0] != 1 or attention_mask.shape[1] != Lk:
             raise ValueError(f"attention_mask must be a (1, {Lk}) padding mask over the keys; got {tuple(attention_mask.shape)}")
         keep_k = attention_mask[0] != 0
@@ -246,10 +245,10 @@ class LlamaFlashAttention2TPSP(nn.Module):
         # queries are the last Lq key positions; a single decoding query is always kept (as the host's unpad does)
         idx_q = idx_k.new_zeros(1) if Lq == 1 else keep_k[Lk - Lq:].nonzero().squeeze(1)
         if idx_k.numel() == Lk and idx_q.numel() == Lq:
-            return ops.flash_attn_func(q, k, v, 0.0, softmax_scale=scale, causal=True)
+            return ops.flash_attn_func(q, k, v, dropout, softmax_scale=scale, causal=True)
         if idx_q.numel() == 0 or idx_k.numel() == 0:
             return q * 0
-        o = ops.flash_attn_func(q.index_select(1, idx_q), k.index_select(1, idx_k), v.index_select(1, idx_k), 0.0,
+        o = ops.flash_attn_func(q.index_select(1, idx_q), k.index_select(1, idx_k), v.index_select(1, idx_k), dropout,
                                 softmax_scale=scale, causal=True)
         return torch.zeros_like(q).index_copy(1, idx_q, o)
 

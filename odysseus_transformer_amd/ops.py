@@ -70,9 +70,21 @@ def _blhd(t: torch.Tensor, name: str) -> Tuple[int, int, int]:
 
 
 # --------------------------------------------------------------------------- attention
-def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=None):
-    """q (B, Lq, Hq, D), k/v (B, Lk, Hkv, D) -> out (B, Lq, Hq, D), lse (B, Hq, Lq) fp32."""
+def _check_dropout(dropout_p: float, seed) -> None:
+    if not 0.0 <= dropout_p < 1.0:
+        raise ValueError(f"dropout_p must be in [0, 1), got {dropout_p}")
+    if dropout_p > 0.0 and seed is None:
+        raise ValueError("attention dropout needs a seed: the backward reproduces the forward's mask from it")
+
+
+def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=None, dropout_p: float = 0.0, seed=None):
+    """q (B, Lq, Hq, D), k/v (B, Lk, Hkv, D) -> out (B, Lq, Hq, D), lse (B, Hq, Lq) fp32.
+
+    dropout_p > 0 (bfloat16 only) drops entries of the softmax matrix before P . V, scaling the kept ones by
+    1 / (1 - dropout_p); which entries is a fixed function of `seed` (an int) and the entry's (batch, head,
+    query, key), so attn_bwd with the same dropout_p and seed sees the same mask.  lse is that of the full P."""
     _need_gpu(q, k, v)
+    _check_dropout(dropout_p, seed)
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
     if k.shape != v.shape or k.shape[0] != B or k.shape[3] != D or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -85,9 +97,13 @@ def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=No
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
     ws_bytes = _lib.load().ody_attn_fwd_workspace_bytes(B, Lq, Lk, Hq, Hkv, D, _dt(q))
     ws = scratch(ws_bytes, "attn_fwd_workspace", q.device) if ws_bytes else None
-    _lib.call("ody_attn_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-              B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
-              scale, int(causal), _dt(q), ws.data_ptr() if ws_bytes else 0, ws_bytes, _stream())
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
+            scale, int(causal), _dt(q), ws.data_ptr() if ws_bytes else 0, ws_bytes, _stream())
+    if dropout_p > 0.0:
+        _lib.call("ody_attn_fwd_dropout", *args, float(dropout_p), int(seed) & 0xFFFFFFFFFFFFFFFF)
+    else:
+        _lib.call("ody_attn_fwd", *args)
     return out, lse
 
 
@@ -112,8 +128,9 @@ def attn_fwd_noalloc(q, k, v, out, lse, causal: bool = True, scale: Optional[flo
 
 def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
              dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False,
-             rope_tables=None, keep_ds: Optional[bool] = None):
-    """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.
+             rope_tables=None, keep_ds: Optional[bool] = None, dropout_p: float = 0.0, seed=None):
+    """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.  dropout_p / seed: those of the
+    forward call (bfloat16; the plain kernels: not with keep_ds=True or rope_tables).
 
     dq may be a float32 tensor although q is bfloat16: with accumulate_dq that is the running dq of a
     ring step, summed exactly over the key blocks.  reuse_query_side=True (needs the `workspace` of
@@ -128,6 +145,11 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
     scratch stays within the budget of set_keep_ds_max_bytes() / ODYSSEUS_KEEP_DS_MAX_BYTES (0 unless set) or is
     already there in the arena; True insists (ValueError where the shape does not qualify); False never."""
     _need_gpu(q, k, v, out, lse, dout)
+    _check_dropout(dropout_p, seed)
+    if dropout_p > 0.0:
+        if keep_ds or rope_tables is not None:
+            raise ValueError("attention dropout runs on the plain kernels: no keep_ds, no rope_tables")
+        keep_ds = False
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
     if dq is None:
@@ -178,7 +200,9 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
             B, Lq, Lk, Hq, Hkv, D, *_blhd(q, "q"), *_blhd(k, "k"), *_blhd(v, "v"), *_blhd(out, "out"),
             *_blhd(dout, "dout"), *_blhd(dq, "dq"), *_blhd(dk, "dk"), *_blhd(dv, "dv"),
             scale, int(causal), flags, _dt(q), ws.data_ptr(), ws_bytes, _stream())
-    if rope_tables is None:
+    if dropout_p > 0.0:
+        _lib.call("ody_attn_bwd_dropout", *args, float(dropout_p), int(seed) & 0xFFFFFFFFFFFFFFFF)
+    elif rope_tables is None:
         _lib.call("ody_attn_bwd", *args)
     else:
         tq, tk = rope_tables
@@ -610,10 +634,10 @@ class FlashAttnFunc(torch.autograd.Function):
     """Causal/full attention with GQA over (B, L, H, D) tensors; returns (out, lse)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, softmax_scale, causal):
-        out, lse = attn_fwd(q, k, v, causal=causal, scale=softmax_scale)
+    def forward(ctx, q, k, v, softmax_scale, causal, dropout_p=0.0, seed=None):
+        out, lse = attn_fwd(q, k, v, causal=causal, scale=softmax_scale, dropout_p=dropout_p, seed=seed)
         ctx.save_for_backward(q, k, v, out, lse)
-        ctx.softmax_scale, ctx.causal = softmax_scale, causal
+        ctx.softmax_scale, ctx.causal, ctx.dropout = softmax_scale, causal, (dropout_p, seed)
         ctx.mark_non_differentiable(lse)
         return out, lse
 
@@ -622,8 +646,9 @@ class FlashAttnFunc(torch.autograd.Function):
         q, k, v, out, lse = ctx.saved_tensors
         if dout.stride(3) != 1:
             dout = dout.contiguous()
-        dq, dk, dv = attn_bwd(q, k, v, out, lse, dout, causal=ctx.causal, scale=ctx.softmax_scale)
-        return dq, dk, dv, None, None
+        dq, dk, dv = attn_bwd(q, k, v, out, lse, dout, causal=ctx.causal, scale=ctx.softmax_scale,
+                              dropout_p=ctx.dropout[0], seed=ctx.dropout[1])
+        return dq, dk, dv, None, None, None, None
 
 
 class RingBlocksAttnFunc(torch.autograd.Function):
@@ -765,14 +790,15 @@ def zigzag_ring_rank_attn(q, k_blocks, v_blocks, rank: int, world_size: int, sof
 
 
 def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[float] = None, causal: bool = False,
-                    return_lse: bool = False):
+                    return_lse: bool = False, seed: Optional[int] = None):
     """Signature of the routine the reference reaches at decoder/odysseus.py:256-263.
 
-    Dropout is not implemented (the training loop of the reference runs with
-    attention_dropout = 0.0); a non-zero value raises."""
-    if dropout_p != 0.0:
-        raise NotImplementedError("attention dropout is not implemented (the reference runs with 0.0)")
-    out, lse = FlashAttnFunc.apply(q, k, v, softmax_scale, causal)
+    dropout_p > 0 (bfloat16): the mask's seed is `seed`, or one drawn from torch's default CPU generator, so that
+    torch.manual_seed makes runs repeatable; the backward reproduces the mask from it.  (The reference's routine draws
+    its masks from a generator of its own: the masks differ, their distribution and the arithmetic do not.)"""
+    if dropout_p != 0.0 and seed is None:
+        seed = int(torch.randint(0, 1 << 62, (1,)).item())
+    out, lse = FlashAttnFunc.apply(q, k, v, softmax_scale, causal, float(dropout_p), seed)
     return (out, lse) if return_lse else out
 
 

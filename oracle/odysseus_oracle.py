@@ -37,6 +37,13 @@ How each function is pinned (tests/test_oracle.py):
                      both moments); with zero gradient only the weight decay acts
   attention_block,   autograd of the composed functions vs. the explicit
   decoder_layer_*    backward formulas in this file
+  dropout (the       given a mask: attention_fwd / attention_bwd == autograd through the brute-force softmax with
+  dropout_p, seed    the same mask applied as torch.nn.functional.dropout does (fp64); p = 0 is the undropped
+  arguments)         result; the kept fraction of dropout_keep_mask is 1 - p within sampling error, and it is the
+                     same for every way of slicing the index ranges.  The mask ITSELF (dropout_keep_mask) is this
+                     build's own counter hash: the reference's routine draws from flash-attn's Philox stream, which
+                     nothing here can reproduce -- the mask's bit pattern is parity-unpinned, its distribution and
+                     the arithmetic are not
 
 Parity unpinned (nothing in the reference, its tests, or mathematics fixes it):
 the exact bf16 rounding sequence of flash-attn's CUDA kernels (P rounded to
@@ -122,9 +129,41 @@ def _ct(t: torch.Tensor) -> torch.dtype:
     return torch.float64 if t.dtype == torch.float64 else torch.float32
 
 
+_M32 = 0xFFFFFFFF
+
+
+def _mix32(x: torch.Tensor) -> torch.Tensor:
+    """The 32-bit finalizer of MurmurHash3 on int64 tensors holding unsigned 32-bit values."""
+    x = x ^ (x >> 16)
+    x = (x * 0x85EBCA6B) & _M32
+    x = x ^ (x >> 13)
+    x = (x * 0xC2B2AE35) & _M32
+    return x ^ (x >> 16)
+
+
+def dropout_keep_mask(seed: int, p_drop: float, B: int, Hq: int, q_idx: torch.Tensor, k_idx: torch.Tensor) -> torch.Tensor:
+    """Which entries of P survive dropout: bool (B, Hq, len(q_idx), len(k_idx)).  The decision for (b, h, q, k) is a
+    fixed function of the seed and the four indices (a counter hash: no state, any kernel can evaluate any entry):
+        u = mix(seed32 ^ (b * Hq + h) * 0x85ebca77);  r = mix(u + q * 0x9e3779b1);  x = mix(r ^ k * 0xc2b2ae3d)
+    kept iff x >= p_drop * 2^32 (all in unsigned 32-bit arithmetic; seed32 = low word ^ high word of the seed)."""
+    seed &= 0xFFFFFFFFFFFFFFFF
+    seed32 = (seed ^ (seed >> 32)) & _M32
+    t = p_drop * 4294967296.0
+    thresh = 4294967295 if t >= 4294967295.0 else (1 if t < 1.0 else int(t))
+    bh = torch.arange(B * Hq, dtype=torch.int64).view(B, Hq, 1, 1)
+    u = _mix32(seed32 ^ ((bh * 0x85EBCA77) & _M32))
+    r = _mix32((u + ((q_idx.to(torch.int64).view(1, 1, -1, 1) * 0x9E3779B1) & _M32)) & _M32)
+    x = _mix32(r ^ ((k_idx.to(torch.int64).view(1, 1, 1, -1) * 0xC2B2AE3D) & _M32))
+    return x >= thresh
+
+
 def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool = True,
-                  scale: Optional[float] = None, block: int = 1024) -> Tuple[torch.Tensor, torch.Tensor]:
+                  scale: Optional[float] = None, block: int = 1024, dropout_p: float = 0.0,
+                  seed: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
     """q (B, Lq, Hq, D), k/v (B, Lk, Hkv, D) -> out (B, Lq, Hq, D), lse (B, Hq, Lq).
+
+    dropout_p > 0 (the dropout_p of the routine called at decoder/odysseus.py:256-263): entries of P are dropped
+    per dropout_keep_mask and the kept ones scaled by 1 / (1 - dropout_p) before P . V; lse is that of the full P.
 
     Causal masking is aligned to the bottom-right corner (key j visible to
     query i iff j <= i + Lk - Lq), which for Lq == Lk is j <= i.  Computed one
@@ -153,14 +192,18 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: boo
             s = s.masked_fill(jj > ii, NEG_INF)
         l = torch.logsumexp(s, dim=-1)                                  # -inf for empty rows
         p = torch.exp(s - torch.where(torch.isinf(l), torch.zeros_like(l), l)[..., None])
+        if dropout_p > 0.0:
+            keep = dropout_keep_mask(seed, dropout_p, B, Hq, torch.arange(i0, i1), torch.arange(kend))
+            p = torch.where(keep, p / (1.0 - dropout_p), torch.zeros_like(p))
         out[:, :, i0:i1] = torch.matmul(p, vh[:, :, :kend])
         lse[:, :, i0:i1] = l
     return out.permute(0, 2, 1, 3).contiguous().to(q.dtype), lse
 
 
 def attention_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float] = None,
-                  block: int = 1024):
-    """Explicit flash-attention backward: returns (dq, dk, dv).
+                  block: int = 1024, dropout_p: float = 0.0, seed: int = 0):
+    """Explicit flash-attention backward: returns (dq, dk, dv).  With dropout (mask M, scale c = 1 / (1 - p)):
+    dV = (c M P)^T dO, dP = c M (dO V^T), and delta, dS, dQ, dK as below.
 
     P = exp(S - lse), dV = P^T dO, dP = dO V^T, delta_i = sum_d dO_id O_id,
     dS = P * (dP - delta), dQ = dS K * scale, dK = dS^T Q * scale; dK and dV of
@@ -194,8 +237,13 @@ def attention_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[
             s = s.masked_fill(jj > ii, NEG_INF)
         l = lse[:, :, i0:i1]
         p = torch.exp(s - torch.where(torch.isinf(l), torch.zeros_like(l), l)[..., None])
-        dv[:, :, :kend] += torch.matmul(p.transpose(-1, -2), doh[:, :, i0:i1])
         dp = torch.matmul(doh[:, :, i0:i1], vh[:, :, :kend].transpose(-1, -2))
+        pd = p
+        if dropout_p > 0.0:
+            keep = dropout_keep_mask(seed, dropout_p, B, Hq, torch.arange(i0, i1), torch.arange(kend))
+            pd = torch.where(keep, p / (1.0 - dropout_p), torch.zeros_like(p))
+            dp = torch.where(keep, dp / (1.0 - dropout_p), torch.zeros_like(dp))
+        dv[:, :, :kend] += torch.matmul(pd.transpose(-1, -2), doh[:, :, i0:i1])
         ds = p * (dp - delta[:, :, i0:i1, None])
         dq[:, :, i0:i1] = torch.matmul(ds, kh[:, :, :kend]) * scale
         dk[:, :, :kend] += torch.matmul(ds.transpose(-1, -2), qh[:, :, i0:i1]) * scale
@@ -205,8 +253,10 @@ def attention_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[
     return f(dq), f(dk), f(dv)
 
 
-def attention_naive(q, k, v, causal: bool = True, scale: Optional[float] = None):
-    """Differentiable brute force (materialises the scores); small inputs only."""
+def attention_naive(q, k, v, causal: bool = True, scale: Optional[float] = None, keep: Optional[torch.Tensor] = None,
+                    dropout_p: float = 0.0):
+    """Differentiable brute force (materialises the scores); small inputs only.  keep: a bool mask (B, Hq, Lq, Lk) of
+    the entries of P that survive dropout, scaled by 1 / (1 - dropout_p)."""
     B, Lq, Hq, D = q.shape
     Lk, Hkv = k.shape[1], k.shape[2]
     G = Hq // Hkv
@@ -221,6 +271,8 @@ def attention_naive(q, k, v, causal: bool = True, scale: Optional[float] = None)
         s = s.masked_fill(jj > ii, NEG_INF)
     lse = torch.logsumexp(s, dim=-1)
     p = torch.softmax(s, dim=-1)
+    if keep is not None:
+        p = torch.where(keep, p / (1.0 - dropout_p), torch.zeros_like(p))
     return torch.matmul(p, vh).permute(0, 2, 1, 3), lse
 
 

@@ -404,3 +404,44 @@ def test_attention_block_decodes_from_a_kv_cache(dev):
     ps = torch.cat([torch.arange(5, L), torch.tensor([L - 5])])[None]
     y2, _ = oracle.attention_block(xs, w.float(), wo.float(), H, Hkv, D, position_ids=ps)
     assert_parity(y, y2[:, -1:], TOL_BF16, "masked decode step", 1e-3)
+
+
+def test_attention_block_trains_with_attention_dropout(dev):
+    """config.attention_dropout > 0 (decoder/odysseus.py:228 passes it on while training): the module drops entries
+    of P with a seed it draws from torch's generator, and eval mode does not drop."""
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    d, H, Hkv, D, L = 512, 4, 2, 128, 320
+    dt = torch.bfloat16
+    cfg = _config(d, H, Hkv, D, 1024)
+    cfg.attention_dropout = 0.25
+    attn = LlamaFlashAttention2TPSP(cfg, 0).to(dt).to(dev)
+    w = randn(((H + 2 * Hkv) * D, d), 37, std=0.02, dtype=dt)
+    wo = randn((d, H * D), 38, std=0.02, dtype=dt)
+    with torch.no_grad():
+        attn.qkv_proj.weight.copy_(w)
+        attn.o_proj.weight.copy_(wo)
+    x = randn((1, L, d), 39, dtype=dt)
+    attn.eval()
+    y_eval = attn(x.to(dev))[0]
+    y_ref, _ = oracle.attention_block(x.float(), w.float(), wo.float(), H, Hkv, D)
+    assert_parity(y_eval, y_ref, TOL_BF16, "eval mode: no dropout")
+    attn.train()
+    torch.manual_seed(5)
+    seed = int(torch.randint(0, 1 << 62, (1,)).item())
+    torch.manual_seed(5)
+    xg = x.to(dev).requires_grad_(True)
+    y = attn(xg)[0]
+    dy = randn((1, L, d), 40, dtype=dt)
+    y.backward(dy.to(dev))
+    # the oracle's block with the same mask
+    xr = x.float().requires_grad_(True)
+    qr, kr, vr = oracle.split_qkv(oracle.linear_fwd(xr, w.float()), H, Hkv, D)
+    cos, sin = oracle.rope_cos_sin(torch.arange(L)[None], D, 10000.0, torch.float32)
+    qr, kr = oracle.apply_rope(qr, cos, sin), oracle.apply_rope(kr, cos, sin)
+    keep = oracle.dropout_keep_mask(seed, 0.25, 1, H, torch.arange(L), torch.arange(L))
+    o, _ = oracle.attention_naive(qr, kr, vr, causal=True, keep=keep, dropout_p=0.25)
+    yr = oracle.linear_fwd(o.reshape(1, L, H * D), wo.float())
+    yr.backward(dy.float())
+    assert_parity(y, yr.detach(), TOL_BF16, "training mode: dropped")
+    assert rel_err(y, y_eval.float().cpu()) > 0.05
+    assert_parity(xg.grad, xr.grad, TOL_BF16, "dx", 1e-3)

@@ -133,6 +133,52 @@ def test_attention_bwd_vs_autograd(Hq, Hkv, Lq, Lk, causal):
     assert torch.allclose(dv, v.grad, atol=1e-10)
 
 
+@pytest.mark.parametrize("Hq,Hkv,Lq,Lk,causal", [(4, 4, 19, 19, True), (4, 2, 23, 23, True), (4, 1, 9, 14, False),
+                                                 (2, 1, 12, 20, True)])
+def test_attention_with_dropout_vs_autograd(Hq, Hkv, Lq, Lk, causal):
+    """Given the mask, the dropout arithmetic is what autograd makes of softmax -> F.dropout's rule (zero or
+    1 / (1 - p)) -> P V; the mask is the same however the index ranges are cut into blocks."""
+    D, pdrop, seed = 8, 0.3, 0x1234ABCD5678
+    q, k, v = (t.requires_grad_() for t in (r64((2, Lq, Hq, D), 30), r64((2, Lk, Hkv, D), 31), r64((2, Lk, Hkv, D), 32)))
+    do = r64((2, Lq, Hq, D), 33)
+    keep = oracle.dropout_keep_mask(seed, pdrop, 2, Hq, torch.arange(Lq), torch.arange(Lk))
+    # the rule of torch's own dropout on the same mask
+    ones = torch.ones(2, Hq, Lq, Lk, dtype=torch.float64)
+    assert torch.equal(torch.where(keep, ones / (1 - pdrop), 0 * ones), keep * F.dropout(ones, pdrop, training=False) / (1 - pdrop))
+    o, lse = oracle.attention_naive(q, k, v, causal=causal, keep=keep, dropout_p=pdrop)
+    o.backward(do)
+    o2, lse2 = oracle.attention_fwd(q.detach(), k.detach(), v.detach(), causal=causal, block=5, dropout_p=pdrop, seed=seed)
+    assert torch.allclose(o2, o.detach(), atol=1e-10) and torch.allclose(lse2, lse.detach(), atol=1e-10)
+    lse_plain = oracle.attention_fwd(q.detach(), k.detach(), v.detach(), causal=causal)[1]
+    assert torch.allclose(lse2, lse_plain, atol=1e-12)             # lse is that of the full P
+    dq, dk, dv = oracle.attention_bwd(q.detach(), k.detach(), v.detach(), o2, lse2, do, causal=causal, block=7,
+                                      dropout_p=pdrop, seed=seed)
+    assert torch.allclose(dq, q.grad, atol=1e-10)
+    assert torch.allclose(dk, k.grad, atol=1e-10)
+    assert torch.allclose(dv, v.grad, atol=1e-10)
+
+
+def test_dropout_mask_properties():
+    """Kept fraction 1 - p within sampling error, for every (batch, head), row and column alike; different seeds,
+    heads and batches give different masks; a mask does not depend on how its index ranges are sliced."""
+    L = 640
+    for pdrop in (0.05, 0.1, 0.5):
+        m = oracle.dropout_keep_mask(99, pdrop, 2, 3, torch.arange(L), torch.arange(L)).double()
+        se = math.sqrt(pdrop * (1 - pdrop) / (L * L))
+        assert (m.mean((-1, -2)) - (1 - pdrop)).abs().max() < 5 * se
+        row_se = math.sqrt(pdrop * (1 - pdrop) / L)
+        assert (m.mean(-1) - (1 - pdrop)).abs().max() < 6 * row_se and (m.mean(-2) - (1 - pdrop)).abs().max() < 6 * row_se
+        # neighbouring entries are uncorrelated (along keys, along queries, across heads)
+        c = m - (1 - pdrop)
+        for a, b in ((c[..., :-1], c[..., 1:]), (c[..., :-1, :], c[..., 1:, :]), (c[:, 0], c[:, 1]), (c[0], c[1])):
+            assert abs((a * b).mean().item()) < 6 * pdrop * (1 - pdrop) / math.sqrt(a.numel())
+    m = oracle.dropout_keep_mask(99, 0.1, 2, 3, torch.arange(L), torch.arange(L))
+    assert not torch.equal(m, oracle.dropout_keep_mask(100, 0.1, 2, 3, torch.arange(L), torch.arange(L)))
+    part = oracle.dropout_keep_mask(99, 0.1, 2, 3, torch.arange(17, 300), torch.arange(401, 640))
+    assert torch.equal(part, m[:, :, 17:300, 401:640])
+    assert not torch.equal(m, oracle.dropout_keep_mask(99 + (1 << 32), 0.1, 2, 3, torch.arange(L), torch.arange(L)))   # all 64 seed bits count
+
+
 def test_gqa_equals_mha_on_repeated_kv():
     q, k, v, do = r64((1, 15, 4, 8), 34), r64((1, 15, 2, 8), 35), r64((1, 15, 2, 8), 36), r64((1, 15, 4, 8), 37)
     o, lse = oracle.attention_fwd(q, k, v)
