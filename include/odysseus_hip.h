@@ -317,8 +317,8 @@ int ody_attn_bwd_rope(const void* q, const void* k, const void* v, const void* o
  * function of (seed, batch, query head, query, key) -- a 32-bit counter hash, restated on the host in
  * oracle/odysseus_oracle.py -- so the backward reproduces the forward's mask from the same seed.  The reference's
  * routine draws its mask from a Philox stream of its own: masks differ, the distribution and the arithmetic given a
- * mask are the same.  bf16 only, head_dim 64 or 128, on the library's plain kernels (no key split, no kept dS, no
- * rotary tables: ODY_BWD_KEEP_DS is refused); p_drop = 0 is exactly ody_attn_fwd / ody_attn_bwd.  Workspaces as
+ * mask are the same.  bf16 and fp32, head_dim 64 or 128; bf16 on the library's plain kernels (no key split, no kept dS,
+ * no rotary tables: ODY_BWD_KEEP_DS is refused); p_drop = 0 is exactly ody_attn_fwd / ody_attn_bwd.  Workspaces as
  * for those.
  */
 int ody_attn_fwd_dropout(const void* q, const void* k, const void* v, void* out, float* lse,

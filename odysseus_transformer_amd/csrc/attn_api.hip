@@ -37,12 +37,11 @@ int check_tensor(const char* who, const char* name, const void* ptr, const AttnS
 extern "C" size_t ody_attn_fwd_workspace_bytes(int B, int Lq, int Lk, int Hq, int Hkv, int D, int dtype);
 
 namespace {
-// p_drop in (0, 1): the dropout fields of the argument block; 0: none.  bf16 only (the kernels that implement it).
-int set_dropout(const char* who, AttnParams& p, float p_drop, uint64_t seed, int dtype) {
+// p_drop in (0, 1): the dropout fields of the argument block; 0: none
+int set_dropout(const char* who, AttnParams& p, float p_drop, uint64_t seed) {
   ODY_REQUIRE(p_drop >= 0.f && p_drop < 1.f, ODY_ERR_BAD_SHAPE, "%s: the dropout probability must be in [0, 1), got %g", who,
               (double)p_drop);
   if (p_drop == 0.f) return ODY_OK;
-  ODY_REQUIRE(dtype == ODY_BF16, ODY_ERR_UNSUPPORTED, "%s: attention dropout is implemented for bf16 only", who);
   const double t = (double)p_drop * 4294967296.0;
   p.drop_thresh = t >= 4294967295.0 ? 4294967295u : (t < 1.0 ? 1u : (unsigned)t);
   p.drop_seed = (unsigned)(seed ^ (seed >> 32));
@@ -61,7 +60,7 @@ int attn_fwd_impl(const char* who, const void* q, const void* k, const void* v, 
   int rc = check_common(who, B, Lq, Lk, Hq, Hkv, D, dtype);
   if (rc) return rc;
   AttnParams p{};
-  if ((rc = set_dropout(who, p, p_drop, seed, dtype))) return rc;
+  if ((rc = set_dropout(who, p, p_drop, seed))) return rc;
   p.q = q; p.k = k; p.v = v; p.out = out; p.lse = lse;
   p.B = B; p.Lq = Lq; p.Lk = Lk; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv;
   p.causal = causal ? 1 : 0; p.off = Lk - Lq;
@@ -207,7 +206,7 @@ int attn_bwd_impl(const char* who, const void* rope_q, const void* rope_k,
   ODY_REQUIRE((flags & ~(ODY_BWD_ACCUMULATE_DQ | ODY_BWD_DQ_F32 | ODY_BWD_REUSE_QUERY_SIDE | ODY_BWD_KEEP_DS)) == 0, ODY_ERR_UNSUPPORTED,
               "%s: unknown flag bits in %d", who, flags);
   AttnParams p{};
-  if ((rc = set_dropout(who, p, p_drop, seed, dtype))) return rc;
+  if ((rc = set_dropout(who, p, p_drop, seed))) return rc;
   ODY_REQUIRE(p.drop_thresh == 0 || !(flags & ODY_BWD_KEEP_DS), ODY_ERR_UNSUPPORTED,
               "%s: ODY_BWD_KEEP_DS is not available with dropout", who);
   ODY_REQUIRE(p.drop_thresh == 0 || !(rope_q || rope_k), ODY_ERR_UNSUPPORTED, "%s: no rotary tables with dropout", who);

@@ -143,7 +143,9 @@ __device__ __forceinline__ void store_rows(float* dst, const f32x16 (&acc)[D / 3
 // ---------------------------------------------------------------------------------------
 // forward
 // ---------------------------------------------------------------------------------------
-template <int D>
+// DROP (all three kernels): attention dropout (AttnParams::drop_*, ody_dropout_hash): row sums and lse are those of the
+// full P; the entries that enter P V are the kept ones scaled by 1 / (1 - p), and dP counts only where an entry was kept.
+template <int D, bool DROP>
 __global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kernel(const AttnParams p) {
   constexpr int LD = D + 4, NDB = D / 32;
   __shared__ __attribute__((aligned(16))) float Ks[F_TILE * LD];
@@ -166,6 +168,7 @@ __global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kerne
 #pragma unroll
     for (int r = 0; r < 16; r++) o[db][r] = 0.f;
   float m = -INFINITY, l = 0.f;
+  const unsigned drow = DROP ? ody_dropout_row(ody_dropout_head(p.drop_seed, b * p.Hq + h), qi) : 0u;
 
   // last key this lane's query sees, the first query of the wavefront sees, and the
   // key ranges the workgroup and the wavefront have to walk
@@ -214,6 +217,7 @@ __global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kerne
     for (int r = 0; r < 16; r++) {
       s[r] = ody_exp2(s[r] - m_use);
       sum += s[r];
+      if (DROP && ody_dropout_hash(drow, n0 + acc_row(r, g)) < p.drop_thresh) s[r] = 0.f;
     }
     l = l * alpha + sum;
 #pragma unroll
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kerne
   l = half_swap_sum(l);
   if (qi < p.Lq) {
     float* op = static_cast<float*>(p.out) + b * p.so.b + h * p.so.h + (int64_t)qi * p.so.l;
-    store_rows<D>(op, o, g, l > 0.f ? 1.f / l : 0.f, false);
+    store_rows<D>(op, o, g, l > 0.f ? (DROP ? p.drop_scale : 1.f) / l : 0.f, false);
     if (g == 0) p.lse[((int64_t)b * p.Hq + h) * p.Lq + qi] = l > 0.f ? (m + __log2f(l)) * LN2 : -INFINITY;
   }
 }
@@ -232,7 +236,7 @@ __global__ __launch_bounds__(F_THREADS, D == 64 ? 3 : 1) void attn_fwd_f32_kerne
 // ---------------------------------------------------------------------------------------
 // dQ: the wavefront owns 32 queries, keys are streamed
 // ---------------------------------------------------------------------------------------
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnParams p) {
   constexpr int LD = D + 4, NDB = D / 32;
   __shared__ __attribute__((aligned(16))) float Ks[F_TILE * LD];
@@ -255,6 +259,7 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnPa
   const float lse = (qi < p.Lq) ? p.lse[ri] : -INFINITY;
   const float lse2 = lse * ODY_LOG2E;
   const float delta = (qi < p.Lq) ? p.delta[ri] : 0.f;
+  const unsigned drow = DROP ? ody_dropout_row(ody_dropout_head(p.drop_seed, b * p.Hq + h), qi) : 0u;
   // a query with no visible key (lse = -inf) contributes nothing
   const int lim = (lse == -INFINITY) ? -1 : (p.causal ? min(p.Lk - 1, qi + p.off) : p.Lk - 1);
   f32x16 dq[NDB];
@@ -290,7 +295,9 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnPa
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const float pr = (n0 + acc_row(r, g) > lim) ? 0.f : ody_exp2(s[r] - lse2);
-      s[r] = pr * (dp[r] - delta) * p.scale;  // dS^T
+      float dpv = dp[r];
+      if (DROP) dpv = ody_dropout_hash(drow, n0 + acc_row(r, g)) >= p.drop_thresh ? dpv * p.drop_scale : 0.f;
+      s[r] = pr * (dpv - delta) * p.scale;  // dS^T
     }
     tile_t_times_regs<D>(Ks, i, g, s, dq);  // dQ^T += K^T dS^T
   }
@@ -305,7 +312,7 @@ __global__ __launch_bounds__(F_THREADS) void attn_bwd_dq_f32_kernel(const AttnPa
 // WHICH: 0 = dV only, 1 = dK only, 2 = both.  (At head_dim 128 the K and V fragments and both
 // accumulators do not fit the register file together, so dV and dK take a pass each.)
 // ---------------------------------------------------------------------------------------
-template <int D, int WHICH>
+template <int D, int WHICH, bool DROP>
 __global__ __launch_bounds__(F_THREADS, (D == 64 || WHICH == 0) ? 2 : 1) void attn_bwd_dkdv_f32_kernel(const AttnParams p) {
   constexpr int LD = D + 4, NDB = D / 32;
   constexpr bool DO_DV = (WHICH != 1), DO_DK = (WHICH != 0);
@@ -345,6 +352,7 @@ __global__ __launch_bounds__(F_THREADS, (D == 64 || WHICH == 0) ? 2 : 1) void at
     const float* qp = static_cast<const float*>(p.q) + b * p.sq.b + h * p.sq.h;
     const float* dop = static_cast<const float*>(p.dout) + b * p.sdo.b + h * p.sdo.h;
     const int64_t rbase = ((int64_t)b * p.Hq + h) * p.Lq;
+    const unsigned dh = DROP ? ody_dropout_head(p.drop_seed, b * p.Hq + h) : 0u;
     auto fetch = [&](int i0) {
       const int valid = min(F_TILE, p.Lq - i0);
       qr.fetch(qp, p.sq.l, i0, valid, tid);
@@ -388,8 +396,13 @@ __global__ __launch_bounds__(F_THREADS, (D == 64 || WHICH == 0) ? 2 : 1) void at
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const float pr = (acc_row(r, g) < vis) ? 0.f : ody_exp2(s[r] - lv[r >> 2][r & 3]);
-        s[r] = pr;
-        if constexpr (DO_DK) dp[r] = pr * (dp[r] - dl[r >> 2][r & 3]) * p.scale;  // dS
+        bool keep = true;
+        if (DROP) keep = ody_dropout_hash(ody_dropout_row(dh, i0 + acc_row(r, g)), ki) >= p.drop_thresh;
+        s[r] = DROP ? (keep ? pr * p.drop_scale : 0.f) : pr;
+        if constexpr (DO_DK) {
+          const float dpv = DROP ? (keep ? dp[r] * p.drop_scale : 0.f) : dp[r];
+          dp[r] = pr * (dpv - dl[r >> 2][r & 3]) * p.scale;  // dS
+        }
       }
       if constexpr (DO_DV) tile_t_times_regs<D>(Os, i, g, s, dv);   // dV^T += dO^T P
       if constexpr (DO_DK) tile_t_times_regs<D>(Qs, i, g, dp, dk);  // dK^T += Q^T dS
@@ -433,28 +446,28 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnParams p) {
   if (row < total && sub == 0) p.delta[row] = acc;
 }
 
-template <int D>
+template <int D, bool DROP>
 int launch_fwd(const AttnParams& p, hipStream_t st) {
   const int nqb = (p.Lq + F_ROWS - 1) / F_ROWS;
-  ODY_LAUNCH("attn_fwd_f32", st, (attn_fwd_f32_kernel<D>), dim3(nqb * p.Hq * p.B), dim3(F_THREADS), 0, p);
+  ODY_LAUNCH("attn_fwd_f32", st, (attn_fwd_f32_kernel<D, DROP>), dim3(nqb * p.Hq * p.B), dim3(F_THREADS), 0, p);
   return ody_check_launch("attn_fwd_f32");
 }
 
-template <int D>
+template <int D, bool DROP>
 int launch_bwd(const AttnParams& p, hipStream_t st) {
   const int nqb = (p.Lq + F_ROWS - 1) / F_ROWS, nkb = (p.Lk + F_ROWS - 1) / F_ROWS;
   const dim3 gk(nkb * p.Hkv * p.B), blk(F_THREADS);
   int rc;
   if constexpr (D == 64) {
-    ODY_LAUNCH("attn_bwd_dkdv_f32", st, (attn_bwd_dkdv_f32_kernel<D, 2>), gk, blk, 0, p);
+    ODY_LAUNCH("attn_bwd_dkdv_f32", st, (attn_bwd_dkdv_f32_kernel<D, 2, DROP>), gk, blk, 0, p);
     if ((rc = ody_check_launch("attn_bwd_dkdv_f32"))) return rc;
   } else {
-    ODY_LAUNCH("attn_bwd_dv_f32", st, (attn_bwd_dkdv_f32_kernel<D, 0>), gk, blk, 0, p);
+    ODY_LAUNCH("attn_bwd_dv_f32", st, (attn_bwd_dkdv_f32_kernel<D, 0, DROP>), gk, blk, 0, p);
     if ((rc = ody_check_launch("attn_bwd_dv_f32"))) return rc;
-    ODY_LAUNCH("attn_bwd_dk_f32", st, (attn_bwd_dkdv_f32_kernel<D, 1>), gk, blk, 0, p);
+    ODY_LAUNCH("attn_bwd_dk_f32", st, (attn_bwd_dkdv_f32_kernel<D, 1, DROP>), gk, blk, 0, p);
     if ((rc = ody_check_launch("attn_bwd_dk_f32"))) return rc;
   }
-  ODY_LAUNCH("attn_bwd_dq_f32", st, (attn_bwd_dq_f32_kernel<D>), dim3(nqb * p.Hq * p.B), blk, 0, p);
+  ODY_LAUNCH("attn_bwd_dq_f32", st, (attn_bwd_dq_f32_kernel<D, DROP>), dim3(nqb * p.Hq * p.B), blk, 0, p);
   return ody_check_launch("attn_bwd_dq_f32");
 }
 
@@ -469,15 +482,17 @@ int launch_delta(const AttnParams& p, hipStream_t st) {
 }  // namespace
 
 int ody_launch_attn_fwd_f32(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 64) return launch_fwd<64>(p, st);
-  if (D == 128) return launch_fwd<128>(p, st);
+  const bool drop = p.drop_thresh != 0;
+  if (D == 64) return drop ? launch_fwd<64, true>(p, st) : launch_fwd<64, false>(p, st);
+  if (D == 128) return drop ? launch_fwd<128, true>(p, st) : launch_fwd<128, false>(p, st);
   ody_set_error("fp32 attention: head_dim %d not built", D);
   return ODY_ERR_UNSUPPORTED;
 }
 
 int ody_launch_attn_bwd_f32(const AttnParams& p, int D, hipStream_t st) {
-  if (D == 64) return launch_bwd<64>(p, st);
-  if (D == 128) return launch_bwd<128>(p, st);
+  const bool drop = p.drop_thresh != 0;
+  if (D == 64) return drop ? launch_bwd<64, true>(p, st) : launch_bwd<64, false>(p, st);
+  if (D == 128) return drop ? launch_bwd<128, true>(p, st) : launch_bwd<128, false>(p, st);
   ody_set_error("fp32 attention: head_dim %d not built", D);
   return ODY_ERR_UNSUPPORTED;
 }

@@ -80,7 +80,7 @@ def _check_dropout(dropout_p: float, seed) -> None:
 def attn_fwd(q, k, v, causal: bool = True, scale: Optional[float] = None, out=None, dropout_p: float = 0.0, seed=None):
     """q (B, Lq, Hq, D), k/v (B, Lk, Hkv, D) -> out (B, Lq, Hq, D), lse (B, Hq, Lq) fp32.
 
-    dropout_p > 0 (bfloat16 only) drops entries of the softmax matrix before P . V, scaling the kept ones by
+    dropout_p > 0 drops entries of the softmax matrix before P . V, scaling the kept ones by
     1 / (1 - dropout_p); which entries is a fixed function of `seed` (an int) and the entry's (batch, head,
     query, key), so attn_bwd with the same dropout_p and seed sees the same mask.  lse is that of the full P."""
     _need_gpu(q, k, v)
@@ -130,7 +130,7 @@ def attn_bwd(q, k, v, out, lse, dout, causal: bool = True, scale: Optional[float
              dq=None, dk=None, dv=None, accumulate_dq: bool = False, workspace=None, reuse_query_side: bool = False,
              rope_tables=None, keep_ds: Optional[bool] = None, dropout_p: float = 0.0, seed=None):
     """Gradients of attn_fwd.  `out`/`lse` may be the merged results of a ring step.  dropout_p / seed: those of the
-    forward call (bfloat16; the plain kernels: not with keep_ds=True or rope_tables).
+    forward call (on the plain kernels: not with keep_ds=True or rope_tables).
 
     dq may be a float32 tensor although q is bfloat16: with accumulate_dq that is the running dq of a
     ring step, summed exactly over the key blocks.  reuse_query_side=True (needs the `workspace` of
@@ -793,7 +793,7 @@ def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[flo
                     return_lse: bool = False, seed: Optional[int] = None):
     """Signature of the routine the reference reaches at decoder/odysseus.py:256-263.
 
-    dropout_p > 0 (bfloat16): the mask's seed is `seed`, or one drawn from torch's default CPU generator, so that
+    dropout_p > 0: the mask's seed is `seed`, or one drawn from torch's default CPU generator, so that
     torch.manual_seed makes runs repeatable; the backward reproduces the mask from it.  (The reference's routine draws
     its masks from a generator of its own: the masks differ, their distribution and the arithmetic do not.)"""
     if dropout_p != 0.0 and seed is None:

@@ -455,18 +455,20 @@ def test_attention_fwd_key_split(case, dev):
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
 @pytest.mark.parametrize("case", [(1, 300, 300, 4, 2, 128, True), (2, 257, 700, 2, 2, 128, False), (1, 1100, 1100, 4, 1, 128, True),
                                   (1, 200, 330, 4, 4, 64, True), (1, 96, 96, 2, 1, 64, False)],
                          ids=lambda c: "B%d_Lq%d_Lk%d_H%d_%d_D%d_c%d" % c)
-def test_attention_dropout_fwd_bwd(case, dev):
+def test_attention_dropout_fwd_bwd(case, dtype, dev):
     """Attention dropout (the dropout_p the reference hands to its attention routine, decoder/odysseus.py:228): the
     kernels evaluate the same counter hash as the oracle, so with the same seed they must agree entry for entry;
     lse is that of the undropped softmax; dropout_p = 0 is the ordinary call."""
     from odysseus_transformer_amd import ops
     B, Lq, Lk, Hq, Hkv, D, causal = case
-    print(f"dropout case={case}", flush=True)
+    print(f"dropout case={case} {dtype}", flush=True)
+    tol = TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
     pdrop, seed = 0.2, 0x9E3779B97F4A7C15 + Lq
-    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, D, torch.bfloat16, seed=11 + Lq)
+    q, k, v, do = _inputs(B, Lq, Lk, Hq, Hkv, D, dtype, seed=11 + Lq)
     o_ref, lse_ref = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal, dropout_p=pdrop, seed=seed)
     dq_ref, dk_ref, dv_ref = oracle.attention_bwd(q.float(), k.float(), v.float(), o_ref, lse_ref, do.float(), causal=causal,
                                                   dropout_p=pdrop, seed=seed)
@@ -475,18 +477,18 @@ def test_attention_dropout_fwd_bwd(case, dev):
     qg, kg, vg, dog = (t.to(dev) for t in (q, k, v, do))
     o, lse = ops.attn_fwd(qg, kg, vg, causal=causal, dropout_p=pdrop, seed=seed)
     dq, dk, dv = ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dropout_p=pdrop, seed=seed)
-    assert_parity(o, o_ref, TOL_BF16, "o")
+    assert_parity(o, o_ref, tol, "o")
     assert torch.allclose(lse.cpu(), lse_ref, atol=TOL_LSE, rtol=TOL_LSE)
-    assert_parity(dq, dq_ref, TOL_BF16, "dq", 1e-3)
-    assert_parity(dk, dk_ref, TOL_BF16, "dk", 1e-3)
-    assert_parity(dv, dv_ref, TOL_BF16, "dv", 1e-3)
+    assert_parity(dq, dq_ref, tol, "dq", 1e-3)
+    assert_parity(dk, dk_ref, tol, "dk", 1e-3)
+    assert_parity(dv, dv_ref, tol, "dv", 1e-3)
     # another seed is another mask; the running fp32 dq of a ring step takes the dropout path too
     o2, _ = ops.attn_fwd(qg, kg, vg, causal=causal, dropout_p=pdrop, seed=seed + 1)
     assert rel_err(o2, o.float().cpu()) > 0.1
     acc0 = randn((B, Lq, Hq, D), 5).to(dev)
     acc = acc0.clone()
     ops.attn_bwd(qg, kg, vg, o, lse, dog, causal=causal, dq=acc, accumulate_dq=True, dropout_p=pdrop, seed=seed)
-    assert_parity((acc - acc0).cpu(), dq_ref, TOL_BF16, "dq added to an fp32 buffer", 1e-3)
+    assert_parity((acc - acc0).cpu(), dq_ref, 4 * tol if dtype == torch.float32 else tol, "dq added to an fp32 buffer", 1e-3)
     # through autograd, with the seed drawn from torch's generator
     qa, ka, va = (t.clone().requires_grad_(True) for t in (qg, kg, vg))
     torch.manual_seed(77)
@@ -496,10 +498,10 @@ def test_attention_dropout_fwd_bwd(case, dev):
     oa.backward(dog)
     o3, lse3 = oracle.attention_fwd(q.float(), k.float(), v.float(), causal=causal, dropout_p=pdrop, seed=drawn)
     dq3, dk3, dv3 = oracle.attention_bwd(q.float(), k.float(), v.float(), o3, lse3, do.float(), causal=causal, dropout_p=pdrop, seed=drawn)
-    assert_parity(oa, o3, TOL_BF16, "o through autograd")
-    assert_parity(qa.grad, dq3, TOL_BF16, "dq through autograd", 1e-3)
-    assert_parity(ka.grad, dk3, TOL_BF16, "dk through autograd", 1e-3)
-    assert_parity(va.grad, dv3, TOL_BF16, "dv through autograd", 1e-3)
+    assert_parity(oa, o3, tol, "o through autograd")
+    assert_parity(qa.grad, dq3, tol, "dq through autograd", 1e-3)
+    assert_parity(ka.grad, dk3, tol, "dk through autograd", 1e-3)
+    assert_parity(va.grad, dv3, tol, "dv through autograd", 1e-3)
 
 
 def test_attention_dropout_errors(dev):
@@ -512,9 +514,11 @@ def test_attention_dropout_errors(dev):
     o, lse = ops.attn_fwd(q, k, v, dropout_p=0.1, seed=1)
     with pytest.raises(ValueError):
         ops.attn_bwd(q, k, v, o, lse, do, dropout_p=0.1, seed=1, keep_ds=True)
-    with pytest.raises(_lib.OdysseusHipError) as e:               # fp32 has no dropout kernels
-        ops.attn_fwd(q.float(), k.float(), v.float(), dropout_p=0.1, seed=1)
-    assert e.value.code == -2
+    with pytest.raises(_lib.OdysseusHipError) as e:               # the C ABI checks the probability itself
+        _lib.call("ody_attn_fwd_dropout", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), 1, 256, 256, 2, 2, 128,
+                  *ops._blhd(q, "q"), *ops._blhd(k, "k"), *ops._blhd(v, "v"), *ops._blhd(o, "o"), 0.088, 1, _lib.ODY_BF16, 0, 0, 0,
+                  1.5, 1)
+    assert e.value.code == -1
     o0, lse0 = ops.attn_fwd(q, k, v, dropout_p=0.0)
     o1, lse1 = ops.attn_fwd(q, k, v)
     assert torch.equal(o0, o1) and torch.equal(lse0, lse1)
