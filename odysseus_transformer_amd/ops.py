@@ -795,7 +795,8 @@ def flash_attn_func(q, k, v, dropout_p: float = 0.0, softmax_scale: Optional[flo
 
     dropout_p > 0: the mask's seed is `seed`, or one drawn from torch's default CPU generator, so that
     torch.manual_seed makes runs repeatable; the backward reproduces the mask from it.  (The reference's routine draws
-    its masks from a generator of its own: the masks differ, their distribution and the arithmetic do not.)"""
+    its masks from a generator of its own: the masks differ, their distribution and the arithmetic do not.)  The seed is
+    a host value: a captured graph replays the mask it was captured with -- pass `seed` per step there."""
     if dropout_p != 0.0 and seed is None:
         seed = int(torch.randint(0, 1 << 62, (1,)).item())
     out, lse = FlashAttnFunc.apply(q, k, v, softmax_scale, causal, float(dropout_p), seed)
