@@ -351,3 +351,75 @@ def test_adamw_host_side():
     p.grad = torch.ones(4)
     with _pytest.raises(RuntimeError, match="no CPU implementation"):
         opt.step()
+
+
+def test_general_attention_path_gathers_and_scatters_like_the_host(monkeypatch):
+    """The host logic of the attention module's general path (padding mask, earlier cache content) on the CPU, with
+    the kernel call replaced by the oracle's brute-force attention: masked tokens take part on neither side, the
+    queries sit at the end of the keys, rows of masked queries are zero, a lone decoding query is always kept
+    (decoder/odysseus.py:215-263 through the host's unpad / varlen / pad)."""
+    import math
+    from transformers import DynamicCache
+    from oracle import odysseus_oracle as oracle
+    from odysseus_transformer_amd import ops
+    from odysseus_transformer_amd.decoder.odysseus import LlamaFlashAttention2TPSP
+    seen = []
+
+    def brute(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, **kw):
+        seen.append((q.shape[1], k.shape[1]))
+        return oracle.attention_naive(q.double(), k.double(), v.double(), causal=causal, scale=softmax_scale)[0].to(q.dtype)
+    monkeypatch.setattr(ops, "flash_attn_func", brute)
+    m = LlamaFlashAttention2TPSP(_cfg(), 0)
+    nh, nkv, D = m.n_local_heads, m.n_local_kv_heads, m.head_dim
+    scale = 1.0 / math.sqrt(D)
+    g = torch.Generator().manual_seed(5)
+
+    def dense(q, k, v, mask):
+        """every query row against all keys, with the mask and the positions written out"""
+        Lq, Lk = q.shape[1], k.shape[1]
+        kh = k.permute(0, 2, 1, 3).repeat_interleave(nh // nkv, dim=1).double()
+        vh = v.permute(0, 2, 1, 3).repeat_interleave(nh // nkv, dim=1).double()
+        s = torch.matmul(q.permute(0, 2, 1, 3).double(), kh.transpose(-1, -2)) * scale
+        pos = torch.arange(Lq)[:, None] + (Lk - Lq)
+        dead = (torch.arange(Lk)[None, :] > pos) | (mask[0] == 0)[None, :]
+        o = torch.matmul(torch.softmax(s.masked_fill(dead, float("-inf")), dim=-1), vh).permute(0, 2, 1, 3)
+        qdead = (mask[0, Lk - Lq:] == 0) if Lq > 1 else torch.zeros(1, dtype=torch.bool)
+        return o.masked_fill(qdead[None, :, None, None], 0.0)
+
+    # prefill with left padding and a hole in the middle
+    L = 24
+    q, k, v = torch.randn(1, L, nh, D, generator=g), torch.randn(1, L, nkv, D, generator=g), torch.randn(1, L, nkv, D, generator=g)
+    mask = torch.ones(1, L, dtype=torch.long)
+    mask[0, :5] = 0
+    mask[0, 11:13] = 0
+    y = m._attend_general(q, k, v, mask, None, None, scale)
+    assert seen[-1] == (L - 7, L - 7)
+    torch.testing.assert_close(y.double(), dense(q, k, v, mask), atol=1e-5, rtol=1e-5)
+    assert torch.count_nonzero(y[0, :5]) == 0 and torch.count_nonzero(y[0, 11:13]) == 0
+    # an all-ones mask and no mask are the plain call
+    y1 = m._attend_general(q, k, v, torch.ones(1, L, dtype=torch.long), None, None, scale)
+    y0 = m._attend_general(q, k, v, None, None, None, scale)
+    assert torch.equal(y0, y1) and seen[-1] == (L, L)
+    with pytest.raises(ValueError, match="padding mask"):
+        m._attend_general(q, k, v, torch.ones(1, L + 1, dtype=torch.long), None, None, scale)
+    # nothing kept: zeros, and no kernel call
+    n = len(seen)
+    assert torch.count_nonzero(m._attend_general(q, k, v, torch.zeros(1, L, dtype=torch.long), None, None, scale)) == 0
+    assert len(seen) == n
+
+    # earlier cache content: 6 new tokens behind the 24 cached ones, the prefill's padding still masked
+    cache = DynamicCache()
+    cache.update(k.transpose(1, 2), v.transpose(1, 2), 0, {})
+    qn, kn, vn = torch.randn(1, 6, nh, D, generator=g), torch.randn(1, 6, nkv, D, generator=g), torch.randn(1, 6, nkv, D, generator=g)
+    mask2 = torch.cat([mask, torch.ones(1, 6, dtype=torch.long)], dim=1)
+    mask2[0, L + 2] = 0
+    y = m._attend_general(qn, kn, vn, mask2, cache, torch.arange(L, L + 6), scale)
+    assert cache.get_seq_length(0) == L + 6 and seen[-1] == (5, L + 6 - 8)
+    k_all, v_all = torch.cat([k, kn], dim=1), torch.cat([v, vn], dim=1)
+    torch.testing.assert_close(y.double(), dense(qn, k_all, v_all, mask2), atol=1e-5, rtol=1e-5)
+    # one decoding token: kept whatever the mask says about it
+    q1, k1, v1 = torch.randn(1, 1, nh, D, generator=g), torch.randn(1, 1, nkv, D, generator=g), torch.randn(1, 1, nkv, D, generator=g)
+    mask3 = torch.cat([mask2, torch.ones(1, 1, dtype=torch.long)], dim=1)
+    y = m._attend_general(q1, k1, v1, mask3, cache, torch.tensor([L + 6]), scale)
+    assert seen[-1] == (1, L + 7 - 8)
+    torch.testing.assert_close(y.double(), dense(q1, torch.cat([k_all, k1], 1), torch.cat([v_all, v1], 1), mask3), atol=1e-5, rtol=1e-5)
